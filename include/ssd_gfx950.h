@@ -1,0 +1,122 @@
+/*
+ * ssd_gfx950.h -- C ABI of libssd_gfx950.so: the Mamba2 SSD chunk-state + state-passing path for
+ * AMD MI355X (gfx950), written as hand-coded HIP kernels.
+ *
+ * Every entry point
+ *   - takes device pointers, element strides and sizes only (no C++ or framework types);
+ *   - enqueues its kernels on the given hipStream_t (passed as void*; NULL = the default stream) and
+ *     returns without synchronising;
+ *   - returns 0 on success, a negative ssd_status for rejected arguments, or a positive hipError_t
+ *     reported by the launch; it never throws and never prints.
+ * Tensors are described by ssd_tensor: a data pointer, an element type and per-dimension strides counted
+ * in elements, so views (for example x and B carved out of a packed projection, or the stride-Q view
+ * dA_cumsum[..., -1]) are passed without copies.  The innermost stride of x, B, states, out,
+ * initial_states and final_states must be 1.
+ *
+ * Replaces, in the reference repository (RishiAstra/mamba-fused-minimal):
+ *   ssd_chunk_state_fwd                -> kernels/ssd_chunk_state.py:202-232 (_chunk_state_fwd) and the
+ *                                         Triton kernel it launches, kernels/ssd_chunk_state.py:97-173
+ *   ssd_state_passing_fwd              -> kernels/ssd_state_passing.py:87-115 (_state_passing_fwd) and
+ *                                         kernels/ssd_state_passing.py:27-84
+ *   ssd_fused_chunk_state_passing_fwd  -> kernels/fused_globalbar.py:201-266 and
+ *                                         kernels/fused_concurrent.py:255-331 (the two fused wrappers used by
+ *                                         main.py:85 and main.py:100) and their kernels
+ */
+#ifndef SSD_GFX950_H
+#define SSD_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SSD_ABI_VERSION 1
+
+typedef enum ssd_dtype {
+    SSD_F32 = 0,
+    SSD_BF16 = 1,
+    SSD_F16 = 2
+} ssd_dtype;
+
+typedef enum ssd_status {
+    SSD_OK = 0,
+    SSD_ERR_NULL = -1,        /* a required pointer is NULL */
+    SSD_ERR_SHAPE = -2,       /* sizes inconsistent (nheads % ngroups, nchunks != ceil(seqlen/chunk), <= 0 ...) */
+    SSD_ERR_DTYPE = -3,       /* element type not supported for this argument */
+    SSD_ERR_STRIDE = -4,      /* innermost stride != 1 where the kernels need it */
+    SSD_ERR_DEVICE = -5,      /* current device is not gfx950, or no device */
+    SSD_ERR_SCRATCH = -6      /* internal scratch could not be obtained */
+} ssd_status;
+
+/* A strided device tensor.  stride[i] is in elements; unused trailing entries are ignored. */
+typedef struct ssd_tensor {
+    void *data;
+    int32_t dtype;            /* ssd_dtype */
+    int32_t reserved;
+    int64_t stride[5];
+} ssd_tensor;
+
+/* Problem sizes.  nchunks must equal ceil(seqlen / chunk_size). */
+typedef struct ssd_dims {
+    int32_t batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks;
+} ssd_dims;
+
+/* ABI version of the loaded library (== SSD_ABI_VERSION it was built with). */
+int ssd_version(void);
+
+/* Static text for a status / hipError_t returned by the calls below. */
+const char *ssd_status_string(int status);
+
+/*
+ * Chunk state (reference: kernels/ssd_chunk_state.py:202-232 / :97-173):
+ *   states[b,c,h,p,n] = sum_{k < lim} x[b,cQ+k,h,p] * B[b,cQ+k,h/(H/G),n] * w_k,
+ *   w_k = exp(min(dA_cumsum[b,h,c,Q-1] - dA_cumsum[b,h,c,k], 0)) * dt[b,h,c,k] * [seq_idx[b,cQ+k] == seq_idx[b,cQ+lim-1]],
+ *   lim = min(Q, seqlen - cQ).
+ * x (b,L,H,P) and B (b,L,G,N): bf16, f16 or f32, same type.  dt, dA_cumsum (b,H,C,Q): f32.
+ * seq_idx (b,L) int32, data == NULL when absent.  states (b,C,H,P,N): f32, bf16 or f16.
+ * clamp != 0 keeps the min(.,0) above (the unfused reference kernel); 0 drops it (the fused reference kernels).
+ */
+int ssd_chunk_state_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                        const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx, const ssd_tensor *states,
+                        const ssd_dims *dims, int clamp, void *stream);
+
+/*
+ * State passing (reference: kernels/ssd_state_passing.py:87-115 / :27-84), on a flattened state axis:
+ *   s = initial_states or 0;  out[:,0] = s;
+ *   for c: s = exp(dA_chunk[b,h,c]) * [id(c) == id(c-1)] * s + states[b,c,h];  out[:,c+1] = s (c < C-1) else final = s
+ *   id(c) = seq_idx[b, min((c+1)Q, seqlen) - 1], id(-1) = 0.
+ * states (b,C,H,dim): f32/bf16/f16.  dA_chunk (b,H,C) f32, any strides.  initial_states (b,H,dim) nullable.
+ * out (b,C,H,dim): f32/bf16/f16.  final_states (b,H,dim): f32.  seqlen and chunk_size are only read when
+ * seq_idx is given.
+ */
+int ssd_state_passing_fwd(const ssd_tensor *states, const ssd_tensor *dA_chunk, const ssd_tensor *initial_states,
+                          const ssd_tensor *seq_idx, const ssd_tensor *out, const ssd_tensor *final_states,
+                          int32_t batch, int32_t nchunks, int32_t nheads, int32_t dim,
+                          int32_t seqlen, int32_t chunk_size, void *stream);
+
+/*
+ * Fused chunk state + state passing in one launch (reference: kernels/fused_globalbar.py:201-266,
+ * kernels/fused_concurrent.py:255-331).  Arguments as in the two calls above, except that
+ * initial_states is (b,H,P,N), out is (b,C,H,P,N), final_states is (b,H,P,N) f32, and the chunk-end decay
+ * is read from dA_cumsum[..., Q-1].  states->data == NULL (or states == NULL) means "do not materialise the
+ * per-chunk states"; otherwise they are written as a side effect exactly as ssd_chunk_state_fwd would.
+ */
+int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                      const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                      const ssd_tensor *initial_states, const ssd_tensor *states,
+                                      const ssd_tensor *out, const ssd_tensor *final_states,
+                                      const ssd_dims *dims, int clamp, void *stream);
+
+/*
+ * Which kernel family the three calls above would pick for these arguments: 1 = bf16 MFMA path,
+ * 0 = generic FMA path (other element types or shapes the MFMA tiling does not cover), negative = rejected.
+ * Pure host logic; launches nothing.
+ */
+int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSD_GFX950_H */

@@ -1,0 +1,188 @@
+// extern "C" entry points of libssd_gfx950.so: argument validation, kernel-family selection, launch.
+#include "../../include/ssd_gfx950.h"
+#include "ssd_params.h"
+
+#include <string.h>
+
+namespace {
+
+using ssd::Params;
+using ssd::PassParams;
+
+bool dtype_ok(int dt) { return dt == SSD_F32 || dt == SSD_BF16 || dt == SSD_F16; }
+
+// Device check, cached per device ordinal: the kernels are gfx950 code objects only.
+int check_device()
+{
+    static int cached[64];      // 0 = unknown, 1 = ok, 2 = not gfx950
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) return SSD_ERR_DEVICE;
+    if (dev < 64 && cached[dev]) return cached[dev] == 1 ? SSD_OK : SSD_ERR_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return SSD_ERR_DEVICE;
+    const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    if (dev < 64) cached[dev] = ok ? 1 : 2;
+    return ok ? SSD_OK : SSD_ERR_DEVICE;
+}
+
+int check_dims(const ssd_dims *d)
+{
+    if (!d) return SSD_ERR_NULL;
+    if (d->batch <= 0 || d->seqlen <= 0 || d->nheads <= 0 || d->headdim <= 0 || d->dstate <= 0 || d->ngroups <= 0 ||
+        d->chunk_size <= 0 || d->nchunks <= 0)
+        return SSD_ERR_SHAPE;
+    if (d->nheads % d->ngroups) return SSD_ERR_SHAPE;
+    if (d->nchunks != (d->seqlen + d->chunk_size - 1) / d->chunk_size) return SSD_ERR_SHAPE;
+    return SSD_OK;
+}
+
+bool present(const ssd_tensor *t) { return t && t->data; }
+
+// Fills the part of Params common to the chunk-state and fused calls.
+int fill_common(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dacs,
+                const ssd_tensor *seq, const ssd_tensor *states, const ssd_dims *d, int clamp)
+{
+    int rc = check_dims(d);
+    if (rc) return rc;
+    if (!present(x) || !present(B) || !present(dt) || !present(dacs)) return SSD_ERR_NULL;
+    if (!dtype_ok(x->dtype) || x->dtype != B->dtype) return SSD_ERR_DTYPE;
+    if (dt->dtype != SSD_F32 || dacs->dtype != SSD_F32) return SSD_ERR_DTYPE;
+    if (x->stride[3] != 1 || B->stride[3] != 1) return SSD_ERR_STRIDE;
+    memset(&p, 0, sizeof(p));
+    p.x = x->data; p.B = B->data; p.dt = (const float *)dt->data; p.dacs = (const float *)dacs->data;
+    p.batch = d->batch; p.seqlen = d->seqlen; p.nheads = d->nheads; p.headdim = d->headdim; p.dstate = d->dstate;
+    p.ngroups = d->ngroups; p.Q = d->chunk_size; p.C = d->nchunks;
+    p.sx_b = x->stride[0]; p.sx_l = x->stride[1]; p.sx_h = x->stride[2];
+    p.sB_b = B->stride[0]; p.sB_l = B->stride[1]; p.sB_g = B->stride[2];
+    p.sdt_b = dt->stride[0]; p.sdt_h = dt->stride[1]; p.sdt_c = dt->stride[2]; p.sdt_k = dt->stride[3];
+    p.sda_b = dacs->stride[0]; p.sda_h = dacs->stride[1]; p.sda_c = dacs->stride[2]; p.sda_k = dacs->stride[3];
+    p.dt_in = x->dtype;
+    p.clamp = clamp ? 1 : 0;
+    if (present(seq)) {
+        p.seq = (const int32_t *)seq->data;
+        p.ssq_b = seq->stride[0]; p.ssq_l = seq->stride[1];
+    }
+    if (present(states)) {
+        if (!dtype_ok(states->dtype)) return SSD_ERR_DTYPE;
+        if (states->stride[4] != 1) return SSD_ERR_STRIDE;
+        p.states = states->data; p.dt_states = states->dtype;
+        p.sst_b = states->stride[0]; p.sst_c = states->stride[1]; p.sst_h = states->stride[2]; p.sst_p = states->stride[3];
+    }
+    return SSD_OK;
+}
+
+int run(const Params &p, bool fused, void *stream)
+{
+    int rc = check_device();
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
+    return (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ssd_version(void) { return SSD_ABI_VERSION; }
+
+const char *ssd_status_string(int status)
+{
+    switch (status) {
+        case SSD_OK: return "ok";
+        case SSD_ERR_NULL: return "a required pointer is NULL";
+        case SSD_ERR_SHAPE: return "inconsistent problem sizes";
+        case SSD_ERR_DTYPE: return "unsupported element type";
+        case SSD_ERR_STRIDE: return "innermost stride must be 1";
+        case SSD_ERR_DEVICE: return "no gfx950 device is current";
+        case SSD_ERR_SCRATCH: return "internal scratch unavailable";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+int ssd_chunk_state_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                        const ssd_tensor *seq_idx, const ssd_tensor *states, const ssd_dims *dims, int clamp,
+                        void *stream)
+{
+    if (!present(states)) return SSD_ERR_NULL;
+    Params p;
+    int rc = fill_common(p, x, B, dt, dA_cumsum, seq_idx, states, dims, clamp);
+    if (rc) return rc;
+    return run(p, false, stream);
+}
+
+int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                      const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                      const ssd_tensor *initial_states, const ssd_tensor *states,
+                                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims,
+                                      int clamp, void *stream)
+{
+    if (!present(out) || !present(final_states)) return SSD_ERR_NULL;
+    Params p;
+    int rc = fill_common(p, x, B, dt, dA_cumsum, seq_idx, states, dims, clamp);
+    if (rc) return rc;
+    if (!dtype_ok(out->dtype) || final_states->dtype != SSD_F32) return SSD_ERR_DTYPE;
+    if (out->stride[4] != 1 || final_states->stride[3] != 1) return SSD_ERR_STRIDE;
+    p.out = out->data; p.dt_out = out->dtype;
+    p.so_b = out->stride[0]; p.so_c = out->stride[1]; p.so_h = out->stride[2]; p.so_p = out->stride[3];
+    p.fin = (float *)final_states->data;
+    p.sf_b = final_states->stride[0]; p.sf_h = final_states->stride[1]; p.sf_p = final_states->stride[2];
+    if (present(initial_states)) {
+        if (!dtype_ok(initial_states->dtype)) return SSD_ERR_DTYPE;
+        if (initial_states->stride[3] != 1) return SSD_ERR_STRIDE;
+        p.init = initial_states->data; p.dt_init = initial_states->dtype;
+        p.sin_b = initial_states->stride[0]; p.sin_h = initial_states->stride[1]; p.sin_p = initial_states->stride[2];
+    }
+    return run(p, true, stream);
+}
+
+int ssd_state_passing_fwd(const ssd_tensor *states, const ssd_tensor *dA_chunk, const ssd_tensor *initial_states,
+                          const ssd_tensor *seq_idx, const ssd_tensor *out, const ssd_tensor *final_states,
+                          int32_t batch, int32_t nchunks, int32_t nheads, int32_t dim, int32_t seqlen,
+                          int32_t chunk_size, void *stream)
+{
+    if (!present(states) || !present(dA_chunk) || !present(out) || !present(final_states)) return SSD_ERR_NULL;
+    if (batch <= 0 || nchunks <= 0 || nheads <= 0 || dim <= 0) return SSD_ERR_SHAPE;
+    if (!dtype_ok(states->dtype) || !dtype_ok(out->dtype) || dA_chunk->dtype != SSD_F32 || final_states->dtype != SSD_F32)
+        return SSD_ERR_DTYPE;
+    if (states->stride[3] != 1 || out->stride[3] != 1 || final_states->stride[2] != 1) return SSD_ERR_STRIDE;
+    PassParams p;
+    memset(&p, 0, sizeof(p));
+    p.states = states->data; p.dt_states = states->dtype;
+    p.sst_b = states->stride[0]; p.sst_c = states->stride[1]; p.sst_h = states->stride[2];
+    p.da = (const float *)dA_chunk->data;
+    p.sda_b = dA_chunk->stride[0]; p.sda_h = dA_chunk->stride[1]; p.sda_c = dA_chunk->stride[2];
+    p.out = out->data; p.dt_out = out->dtype;
+    p.so_b = out->stride[0]; p.so_c = out->stride[1]; p.so_h = out->stride[2];
+    p.fin = (float *)final_states->data;
+    p.sf_b = final_states->stride[0]; p.sf_h = final_states->stride[1];
+    p.batch = batch; p.C = nchunks; p.nheads = nheads; p.dim = dim;
+    if (present(initial_states)) {
+        if (!dtype_ok(initial_states->dtype)) return SSD_ERR_DTYPE;
+        if (initial_states->stride[2] != 1) return SSD_ERR_STRIDE;
+        p.init = initial_states->data; p.dt_init = initial_states->dtype;
+        p.sin_b = initial_states->stride[0]; p.sin_h = initial_states->stride[1];
+    }
+    if (present(seq_idx)) {
+        if (seqlen <= 0 || chunk_size <= 0) return SSD_ERR_SHAPE;
+        p.seq = (const int32_t *)seq_idx->data;
+        p.ssq_b = seq_idx->stride[0]; p.ssq_l = seq_idx->stride[1];
+        p.seqlen = seqlen; p.Q = chunk_size;
+    }
+    int rc = check_device();
+    if (rc) return rc;
+    return (int)ssd::launch_state_passing(p, (hipStream_t)stream);
+}
+
+int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims)
+{
+    Params p;
+    ssd_tensor f32 = {(void *)16, SSD_F32, 0, {0, 0, 0, 1, 0}};
+    int rc = fill_common(p, x, B, &f32, &f32, nullptr, nullptr, dims, 1);
+    if (rc) return rc;
+    return ssd::mfma_supported(p) ? 1 : 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,82 @@
+// Internal kernel-argument block shared by the HIP kernels and the C-ABI dispatcher.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ssd {
+
+enum : int { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+
+// All strides are in elements of the tensor they index; innermost strides of x, B, states, out,
+// init and fin are 1 (checked on the host).
+struct Params {
+    const void *x;        // (b, L, H, P)
+    const void *B;        // (b, L, G, N)
+    const float *dt;      // (b, H, C, Q)
+    const float *dacs;    // (b, H, C, Q)
+    const int32_t *seq;   // (b, L) or null
+    const void *init;     // (b, H, P, N) or null
+    void *states;         // (b, C, H, P, N) or null
+    void *out;            // (b, C, H, P, N)           (fused only)
+    float *fin;           // (b, H, P, N)              (fused only)
+    int batch, seqlen, nheads, headdim, dstate, ngroups, Q, C;
+    int64_t sx_b, sx_l, sx_h;
+    int64_t sB_b, sB_l, sB_g;
+    int64_t sdt_b, sdt_h, sdt_c, sdt_k;
+    int64_t sda_b, sda_h, sda_c, sda_k;
+    int64_t ssq_b, ssq_l;
+    int64_t sin_b, sin_h, sin_p;
+    int64_t sst_b, sst_c, sst_h, sst_p;
+    int64_t so_b, so_c, so_h, so_p;
+    int64_t sf_b, sf_h, sf_p;
+    int dt_in, dt_states, dt_out, dt_init;
+    int clamp;
+    int n_items;          // work items of the launch
+};
+
+// State passing on a flattened state axis.
+struct PassParams {
+    const void *states;   // (b, C, H, dim)
+    const float *da;      // (b, H, C)
+    const void *init;     // (b, H, dim) or null
+    const int32_t *seq;   // (b, L) or null
+    void *out;            // (b, C, H, dim)
+    float *fin;           // (b, H, dim)
+    int batch, C, nheads, dim, seqlen, Q;
+    int64_t sst_b, sst_c, sst_h;
+    int64_t sda_b, sda_h, sda_c;
+    int64_t sin_b, sin_h;
+    int64_t ssq_b, ssq_l;
+    int64_t so_b, so_c, so_h;
+    int64_t sf_b, sf_h;
+    int dt_states, dt_out, dt_init;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t hbits) { return __builtin_bit_cast(float, hbits << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
+{
+    return __builtin_bit_cast(uint16_t, (__bf16)f);   // round to nearest even
+}
+
+__device__ __forceinline__ float load_as_f32(const void *base, int64_t idx, int dt)
+{
+    if (dt == DT_F32) return ((const float *)base)[idx];
+    if (dt == DT_BF16) return bf16_bits_to_f32(((const uint16_t *)base)[idx]);
+    return (float)((const _Float16 *)base)[idx];
+}
+
+__device__ __forceinline__ void store_from_f32(void *base, int64_t idx, int dt, float v)
+{
+    if (dt == DT_F32) ((float *)base)[idx] = v;
+    else if (dt == DT_BF16) ((uint16_t *)base)[idx] = f32_to_bf16_bits(v);
+    else ((_Float16 *)base)[idx] = (_Float16)v;
+}
+
+// Launchers implemented in the .hip files; each returns the hipError_t of its launch.
+hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
+hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
+hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
+bool mfma_supported(const Params &p);
+
+}  // namespace ssd

@@ -1,0 +1,9 @@
+"""MI355X (gfx950) implementation of the Mamba2 SSD chunk-state + state-passing path.
+
+Host wrappers with the reference's call surface over hand-written HIP kernels (libssd_gfx950.so, C ABI in
+include/ssd_gfx950.h)."""
+from .ops import (_chunk_state_fwd, _state_passing_fwd, _fused_chunk_state_state_passing_fwd,
+                  _fused_chunk_state_state_passing_fwd_globalbar, _fused_chunk_state_state_passing_fwd_concurrent)
+
+__all__ = ["_chunk_state_fwd", "_state_passing_fwd", "_fused_chunk_state_state_passing_fwd",
+           "_fused_chunk_state_state_passing_fwd_globalbar", "_fused_chunk_state_state_passing_fwd_concurrent"]

@@ -1,0 +1,152 @@
+"""Host-side mirror of the reference call surface for the SSD chunk-state + state-passing path.
+
+Same names, positional order, defaults, shape asserts and output shapes/dtypes as
+  kernels/ssd_chunk_state.py:202-232       _chunk_state_fwd
+  kernels/ssd_state_passing.py:87-115      _state_passing_fwd
+  kernels/fused_globalbar.py:201-266       _fused_chunk_state_state_passing_fwd_globalbar
+  kernels/fused_concurrent.py:255-331      _fused_chunk_state_state_passing_fwd_concurrent
+of the reference.  The wrappers own allocation and argument checking; the arithmetic runs in the gfx950 HIP
+kernels behind the C ABI of libssd_gfx950.so, asynchronously on the current torch stream."""
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
+    # Callers guarantee a unit innermost stride for x and B (main.py:45-54 makes them contiguous otherwise).
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if B.stride(-1) != 1:
+        B = B.contiguous()
+    if B.dtype != x.dtype:
+        B = B.to(x.dtype)
+    if dt.dtype != torch.float32:
+        dt = dt.float()
+    if dA_cumsum.dtype != torch.float32:
+        dA_cumsum = dA_cumsum.float()
+    if seq_idx is not None and seq_idx.dtype != torch.int32:
+        seq_idx = seq_idx.to(torch.int32)
+    return B, x, dt, dA_cumsum, seq_idx
+
+
+def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == dt.shape
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+    if states is not None:
+        assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+    _lib.require_device(x, "_chunk_state_fwd")
+    lib = _lib.load()
+    if states is None:
+        states_dtype = torch.float32 if states_in_fp32 else B.dtype
+        states = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=states_dtype)
+    B, x, dt, dA_cumsum, seq_idx = _prep_inputs(B, x, dt, dA_cumsum, seq_idx)
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    with torch.cuda.device(x.device):
+        rc = lib.ssd_chunk_state_fwd(_lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt),
+                                     _lib.tensor_arg(dA_cumsum), _lib.tensor_arg(seq_idx), _lib.tensor_arg(states),
+                                     dims, 1, _stream(x))
+    _lib.check(rc, "ssd_chunk_state_fwd")
+    return states
+
+
+def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=None, chunk_size=None,
+                       out_dtype=None):
+    batch, nchunks, nheads, dim = states.shape
+    assert dA_chunk_cumsum.shape == (batch, nheads, nchunks)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, dim)
+    seqlen = 0
+    if seq_idx is not None:
+        assert chunk_size is not None
+        seqlen = seq_idx.shape[-1]
+        assert seq_idx.shape == (batch, seqlen)
+    _lib.require_device(states, "_state_passing_fwd")
+    lib = _lib.load()
+    out_dtype = states.dtype if out_dtype is None else out_dtype
+    out = torch.empty((batch, nchunks, nheads, dim), device=states.device, dtype=out_dtype)
+    final_states = torch.empty((batch, nheads, dim), device=states.device, dtype=torch.float32)
+    if states.stride(-1) != 1:
+        states = states.contiguous()
+    if dA_chunk_cumsum.dtype != torch.float32:
+        dA_chunk_cumsum = dA_chunk_cumsum.float()
+    if initial_states is not None and initial_states.stride(-1) != 1:
+        initial_states = initial_states.contiguous()
+    if seq_idx is not None and seq_idx.dtype != torch.int32:
+        seq_idx = seq_idx.to(torch.int32)
+    with torch.cuda.device(states.device):
+        rc = lib.ssd_state_passing_fwd(_lib.tensor_arg(states), _lib.tensor_arg(dA_chunk_cumsum),
+                                       _lib.tensor_arg(initial_states), _lib.tensor_arg(seq_idx),
+                                       _lib.tensor_arg(out), _lib.tensor_arg(final_states),
+                                       batch, nchunks, nheads, dim, seqlen,
+                                       chunk_size if seq_idx is not None else 0, _stream(states))
+    _lib.check(rc, "ssd_state_passing_fwd")
+    return out, final_states
+
+
+def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=None, seq_idx=None,
+                                         states=None, states_in_fp32=True, _clamp=True):
+    """One launch for chunk state + state passing.  Returns (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32).
+
+    Unlike the reference's fused wrappers, the per-chunk states are an internal quantity that never reaches
+    memory unless the caller passes a ``states=`` buffer, which is then filled as a side effect."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum.shape == dt.shape
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+    if states is not None:
+        assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+        states_dtype = states.dtype
+    else:
+        states_dtype = torch.float32 if states_in_fp32 else B.dtype
+    assert dA_cumsum.shape[:3] == (batch, nheads, nchunks)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+    assert chunk_size is not None
+    _lib.require_device(x, "_fused_chunk_state_state_passing_fwd")
+    lib = _lib.load()
+    out_dtype = states_dtype if out_dtype is None else out_dtype
+    out = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=out_dtype)
+    final_states = torch.empty((batch, nheads, headdim, dstate), device=x.device, dtype=torch.float32)
+    B, x, dt, dA_cumsum, seq_idx = _prep_inputs(B, x, dt, dA_cumsum, seq_idx)
+    if initial_states is not None and initial_states.stride(-1) != 1:
+        initial_states = initial_states.contiguous()
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    with torch.cuda.device(x.device):
+        rc = lib.ssd_fused_chunk_state_passing_fwd(
+            _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),
+            _lib.tensor_arg(seq_idx), _lib.tensor_arg(initial_states), _lib.tensor_arg(states),
+            _lib.tensor_arg(out), _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, _stream(x))
+    _lib.check(rc, "ssd_fused_chunk_state_passing_fwd")
+    return out, final_states
+
+
+def _fused_chunk_state_state_passing_fwd_globalbar(B, x, dt, dA_cumsum, out_dtype, initial_states=None,
+                                                   seq_idx=None, states=None, states_in_fp32=True):
+    """Drop-in for kernels/fused_globalbar.py:201 (same signature and returns)."""
+    return _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=initial_states,
+                                                seq_idx=seq_idx, states=states, states_in_fp32=states_in_fp32)
+
+
+def _fused_chunk_state_state_passing_fwd_concurrent(B, x, dt, dA_cumsum, out_dtype, initial_states=None,
+                                                    seq_idx=None, states=None, states_in_fp32=True):
+    """Drop-in for kernels/fused_concurrent.py:255 (same signature and returns; prints nothing)."""
+    return _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=initial_states,
+                                                seq_idx=seq_idx, states=states, states_in_fp32=states_in_fp32)

@@ -1,0 +1,123 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports what include/ssd_gfx950.h
+declares, the wrappers mirror the reference's signatures and assertion behaviour, and nothing silently falls
+back to a CPU computation."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ssd_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("ssd_build", os.path.join(ROOT, "mamba-fused-minimal_amd", "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build_library()
+    return _lib.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "ssd_gfx950.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ssd_[a-z_]+)\s*\(", header))
+    assert {"ssd_version", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd",
+            "ssd_status_string", "ssd_query_path"} <= declared
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.ssd_version() == int(re.search(r"#define SSD_ABI_VERSION (\d+)", header).group(1))
+    from ssd_amd import _lib
+    assert set(_lib.EXPORTS) == declared
+
+
+def test_struct_layouts_match_header():
+    from ssd_amd import _lib
+    assert ctypes.sizeof(_lib.SsdTensor) == 8 + 4 + 4 + 5 * 8
+    assert ctypes.sizeof(_lib.SsdDims) == 8 * 4
+
+
+def test_status_strings_and_argument_rejection_without_gpu(lib):
+    from ssd_amd import _lib
+    assert lib.ssd_status_string(0) == b"ok"
+    x = torch.zeros(1, 256, 2, 64, dtype=torch.bfloat16)
+    B = torch.zeros(1, 256, 1, 128, dtype=torch.bfloat16)
+    dims = _lib.dims_arg(1, 256, 2, 64, 128, 1, 256, 1)
+    assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B), dims) == 1          # MFMA path
+    assert lib.ssd_query_path(_lib.tensor_arg(x.float()), _lib.tensor_arg(B.float()), dims) == 0   # generic path
+    bad = _lib.dims_arg(1, 256, 3, 64, 128, 2, 256, 1)                                     # nheads % ngroups
+    assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B), bad) == -2
+    bad = _lib.dims_arg(1, 256, 2, 64, 128, 1, 256, 2)                                     # wrong nchunks
+    assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B), bad) == -2
+    assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B.float()), dims) == -3  # mixed dtypes
+    xs = x.transpose(2, 3)                                                                 # innermost stride != 1
+    assert lib.ssd_query_path(_lib.tensor_arg(xs), _lib.tensor_arg(B), dims) == -4
+    assert lib.ssd_query_path(_lib.tensor_arg(None), _lib.tensor_arg(B), dims) == -1
+    odd = _lib.dims_arg(1, 256, 2, 40, 128, 1, 256, 1)                                     # headdim 40: generic
+    assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B), odd) == 0
+
+
+def test_signatures_match_reference_call_surface():
+    import ssd_amd
+    sig = lambda f: list(inspect.signature(f).parameters)
+    # kernels/ssd_chunk_state.py:202
+    assert sig(ssd_amd._chunk_state_fwd) == ["B", "x", "dt", "dA_cumsum", "seq_idx", "states", "states_in_fp32"]
+    # kernels/ssd_state_passing.py:87
+    assert sig(ssd_amd._state_passing_fwd) == ["states", "dA_chunk_cumsum", "initial_states", "seq_idx", "chunk_size", "out_dtype"]
+    # kernels/fused_globalbar.py:201, kernels/fused_concurrent.py:255
+    want = ["B", "x", "dt", "dA_cumsum", "out_dtype", "initial_states", "seq_idx", "states", "states_in_fp32"]
+    assert sig(ssd_amd._fused_chunk_state_state_passing_fwd_globalbar) == want
+    assert sig(ssd_amd._fused_chunk_state_state_passing_fwd_concurrent) == want
+    d = inspect.signature(ssd_amd._chunk_state_fwd).parameters
+    assert d["seq_idx"].default is None and d["states"].default is None and d["states_in_fp32"].default is True
+
+
+def test_shape_asserts_mirror_the_reference():
+    import ssd_amd
+    x = torch.zeros(1, 256, 4, 64)
+    B = torch.zeros(1, 256, 1, 128)
+    dt = torch.zeros(1, 4, 1, 256)
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_state_fwd(torch.zeros(1, 256, 3, 128), x, dt, dt)                   # nheads % ngroups
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_state_fwd(B, x, torch.zeros(1, 4, 2, 256), dt)                      # dA_cumsum.shape != dt.shape
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_state_fwd(B, x, dt, dt, seq_idx=torch.zeros(1, 255, dtype=torch.int32))
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_state_fwd(B, x, dt, dt, states=torch.zeros(1, 1, 4, 64, 64))
+    with pytest.raises(AssertionError):
+        ssd_amd._state_passing_fwd(torch.zeros(1, 2, 4, 8), torch.zeros(1, 4, 3))
+    with pytest.raises(AssertionError):
+        ssd_amd._state_passing_fwd(torch.zeros(1, 2, 4, 8), torch.zeros(1, 4, 2), initial_states=torch.zeros(1, 4, 9))
+    with pytest.raises(AssertionError):
+        ssd_amd._state_passing_fwd(torch.zeros(1, 2, 4, 8), torch.zeros(1, 4, 2), seq_idx=torch.zeros(1, 16, dtype=torch.int32))
+    with pytest.raises(AssertionError):
+        ssd_amd._fused_chunk_state_state_passing_fwd_globalbar(B, x, dt, dt, torch.float32,
+                                                               initial_states=torch.zeros(1, 4, 64 * 128))
+
+
+def test_no_cpu_fallback():
+    import ssd_amd
+    x = torch.zeros(1, 256, 4, 64)
+    B = torch.zeros(1, 256, 1, 128)
+    dt = torch.zeros(1, 4, 1, 256)
+    for call in (lambda: ssd_amd._chunk_state_fwd(B, x, dt, dt),
+                 lambda: ssd_amd._state_passing_fwd(torch.zeros(1, 2, 4, 8), torch.zeros(1, 4, 2)),
+                 lambda: ssd_amd._fused_chunk_state_state_passing_fwd_concurrent(B, x, dt, dt, torch.float32)):
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            call()
+
+
+def test_product_code_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "mamba-fused-minimal_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)

@@ -1,0 +1,213 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Tolerance (from the benchmark contract): rtol 2e-3 / atol 1e-3 against an fp32 evaluation, bf16 inputs,
+fp32 states.  bf16 outputs (out_dtype / states_in_fp32=False) are compared at the reference's own
+self-check tolerance rtol 1e-2 / atol 1e-3 (main.py:121)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-3, 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import ssd_amd
+    from ssd_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return ssd_amd
+
+
+def _dev(t):
+    return None if t is None else t.cuda()
+
+
+def _check(name, got, want, rtol=RTOL, atol=ATOL):
+    got = got.float().cpu()
+    want = want.float()
+    assert got.shape == want.shape, (name, got.shape, want.shape)
+    err = (got - want).abs()
+    bad = err > (atol + rtol * want.abs())
+    nbad = int(bad.sum())
+    print(f"[{name}] max_abs={float(err.max()):.3e} max_ref={float(want.abs().max()):.3e} mismatches={nbad}/{want.numel()}",
+          flush=True)
+    assert torch.isfinite(got).all(), name
+    assert nbad == 0, f"{name}: {nbad} mismatches, max abs err {float(err.max()):.3e}"
+
+
+def _run_case(ops, oracle, d, with_states=True, out_dtype=torch.float32, check_unfused=True, name="case"):
+    x, B, dt, dAcs = d["x"], d["B"], d["dt"], d["dA_cumsum"]
+    seq, init = d["seq_idx"], d["initial_states"]
+    print(f"[{name}] x{tuple(x.shape)} {x.dtype} B{tuple(B.shape)} seq={seq is not None} init={init is not None}", flush=True)
+    want_states = oracle.chunk_state_ref(B, x, dt, dAcs, seq_idx=seq)
+    want_out, want_fin = oracle.fused_ref(B, x, dt, dAcs, initial_states=init, seq_idx=seq)
+    xd, Bd, dtd, dAd, seqd, initd = map(_dev, (x, B, dt, dAcs, seq, init))
+    b, L, H, P = x.shape
+    N = B.shape[-1]
+    C = dt.shape[2]
+    # poison the outputs: every element must be written by the kernel
+    st_buf = torch.full((b, C, H, P, N), float("nan"), device="cuda") if with_states else None
+    out, fin = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, out_dtype, initial_states=initd,
+                                                        seq_idx=seqd, states=st_buf)
+    torch.cuda.synchronize()
+    assert out.dtype == out_dtype and fin.dtype == torch.float32
+    assert out.shape == (b, C, H, P, N) and fin.shape == (b, H, P, N)
+    lo = out_dtype != torch.float32
+    _check(name + ".out", out, want_out, *((1e-2, 1e-3) if lo else (RTOL, ATOL)))
+    _check(name + ".final", fin, want_fin)
+    if with_states:
+        _check(name + ".states", st_buf, want_states)
+    if check_unfused:
+        st = ops._chunk_state_fwd(Bd, xd, dtd, dAd, seq_idx=seqd)
+        _check(name + ".chunk_state", st, want_states)
+        o2, f2 = ops._state_passing_fwd(st.flatten(-2), dAd[:, :, :, -1],
+                                        initial_states=None if initd is None else initd.flatten(-2),
+                                        seq_idx=seqd, chunk_size=dt.shape[-1])
+        torch.cuda.synchronize()
+        _check(name + ".state_passing.out", o2.reshape(b, C, H, P, N), want_out)
+        _check(name + ".state_passing.final", f2.reshape(b, H, P, N), want_fin)
+        if with_states and not lo:
+            # the fused kernel and the two unfused kernels share the contraction code: bit-identical states
+            assert torch.equal(st, st_buf)
+    return out, fin
+
+
+# ------------------------------------------------------------------ the five benchmark configurations
+def test_config0_fp32_generic_path(ops, oracle):
+    _run_case(ops, oracle, oracle.make_inputs(0), name="cfg0")
+
+
+def test_config1_mamba2_130m(ops, oracle):
+    _run_case(ops, oracle, oracle.make_inputs(1), name="cfg1")
+
+
+@pytest.mark.timeout(600)
+def test_config2_mamba2_2p7b_with_initial_states(ops, oracle):
+    _run_case(ops, oracle, oracle.make_inputs(2), name="cfg2")
+
+
+@pytest.mark.timeout(600)
+def test_config3_varlen_packed(ops, oracle):
+    d = oracle.make_inputs(3)
+    out, fin = _run_case(ops, oracle, d, name="cfg3")
+    # packed == solo: the final state is the last sequence evaluated alone from a zero state
+    n_last = int(d["seq_lens"][-1])
+    sl = slice(d["x"].shape[1] - n_last, None)
+    hs = [0, 41, 79]
+    o64, f64 = oracle.token_recurrence_ref(d["x"][:, sl][:, :, hs], d["B"][:, sl], d["dt_tok"][:, sl][:, :, hs],
+                                           d["A"][hs], 10 ** 9)
+    _check("cfg3.final_vs_solo_token_recurrence", fin[:, hs], f64)
+
+
+@pytest.mark.timeout(900)
+def test_config4_long_grouped_slicewise(ops, oracle):
+    d = oracle.make_inputs(4)
+    x, B, dt, dAcs = d["x"], d["B"], d["dt"], d["dA_cumsum"]
+    print(f"[cfg4] x{tuple(x.shape)} B{tuple(B.shape)}", flush=True)
+    xd, Bd, dtd, dAd = map(_dev, (x, B, dt, dAcs))
+    out, fin = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32)
+    torch.cuda.synchronize()
+    ratio = x.shape[2] // B.shape[2]
+    for h in (0, 17, 63, 127):                 # one head of four different groups, compared against the oracle
+        g = h // ratio
+        wo, wf = oracle.fused_ref(B[:, :, g:g + 1], x[:, :, h:h + 1], dt[:, h:h + 1], dAcs[:, h:h + 1])
+        _check(f"cfg4.h{h}.out", out[:, :, h:h + 1], wo)
+        _check(f"cfg4.h{h}.final", fin[:, h:h + 1], wf)
+    # full-size property: fused == the library's own unfused kernels, for every head
+    st = ops._chunk_state_fwd(Bd, xd, dtd, dAd)
+    o2, f2 = ops._state_passing_fwd(st.flatten(-2), dAd[:, :, :, -1])
+    torch.cuda.synchronize()
+    assert torch.equal(f2.reshape(fin.shape), fin)
+    assert torch.equal(o2.reshape(out.shape), out)
+
+
+# ------------------------------------------------------------------ shapes, layouts and options beyond the five
+@pytest.mark.parametrize("kw", [
+    dict(L=1000),                                        # ragged last chunk
+    dict(L=1000, nseq=5),                                # ragged + packed sequences
+    dict(Q=128, L=1024),                                 # chunk 128
+    dict(N=64),                                          # dstate 64 on the bf16 MFMA path
+    dict(P=128, H=4),                                    # headdim 128
+    dict(H=8, G=4),                                      # grouped B
+    dict(L=300, H=3, P=40, N=24, G=1, Q=64),             # nothing aligned: generic path
+    dict(dtype="fp16"),                                  # fp16 inputs: generic path
+    dict(b=3, L=256, H=5),                               # a single chunk
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_small_variants(ops, oracle, kw):
+    base = dict(b=2, L=1024, H=6, G=1, init=True)
+    base.update(kw)
+    _run_case(ops, oracle, oracle.make_inputs(1, **base), name="variant")
+
+
+def test_bf16_outputs(ops, oracle):
+    d = oracle.make_inputs(1, b=2, L=1024, H=6, init=True)
+    _run_case(ops, oracle, d, with_states=False, out_dtype=torch.bfloat16, check_unfused=False, name="bf16out")
+    xd, Bd, dtd, dAd = map(_dev, (d["x"], d["B"], d["dt"], d["dA_cumsum"]))
+    st = ops._chunk_state_fwd(Bd, xd, dtd, dAd, states_in_fp32=False)
+    assert st.dtype == torch.bfloat16
+    _check("bf16 states", st, oracle.chunk_state_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"]), 1e-2, 1e-3)
+    o, f = ops._state_passing_fwd(st.flatten(-2), dAd[..., -1], out_dtype=torch.bfloat16)
+    wo, wf = oracle.state_passing_ref(st.cpu().flatten(-2), d["dA_cumsum"][..., -1], out_dtype=torch.bfloat16)
+    _check("bf16 state passing out", o, wo, 1e-2, 1e-3)
+    _check("bf16 state passing final", f, wf)
+
+
+def test_strided_views_of_a_packed_projection(ops, oracle):
+    # x and B carved out of one (b, L, d_inner + 2*G*N) buffer, as a Mamba2 block does: row stride != H*P
+    d = oracle.make_inputs(1, b=2, L=512, H=6)
+    b, L, H, P = d["x"].shape
+    G, N = d["B"].shape[2:]
+    packed = torch.zeros(b, L, H * P + 2 * G * N, dtype=torch.bfloat16, device="cuda")
+    packed[..., :H * P] = d["x"].cuda().reshape(b, L, H * P)
+    packed[..., H * P:H * P + G * N] = d["B"].cuda().reshape(b, L, G * N)
+    xv = packed[..., :H * P].view(b, L, H, P)
+    Bv = packed[..., H * P:H * P + G * N].view(b, L, G, N)
+    assert not xv.is_contiguous()
+    out, fin = ops._fused_chunk_state_state_passing_fwd(Bv, xv, d["dt"].cuda(), d["dA_cumsum"].cuda(), torch.float32)
+    wo, wf = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    _check("strided.out", out, wo)
+    _check("strided.final", fin, wf)
+
+
+def test_back_to_back_launches_are_deterministic(ops, oracle):
+    d = oracle.make_inputs(3, L=8192, H=16, nseq=6)
+    args = list(map(_dev, (d["B"], d["x"], d["dt"], d["dA_cumsum"])))
+    seq = d["seq_idx"].cuda()
+    outs = [ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, seq_idx=seq) for _ in range(4)]
+    torch.cuda.synchronize()
+    for o, f in outs[1:]:
+        assert torch.equal(o, outs[0][0]) and torch.equal(f, outs[0][1])
+
+
+def test_linearity_at_full_size(ops, oracle):
+    # size-independent property at the benchmark shape: scaling x by 2 scales every output by exactly 2
+    d = oracle.make_inputs(2)
+    Bd, xd, dtd, dAd = map(_dev, (d["B"], d["x"], d["dt"], d["dA_cumsum"]))
+    o1, f1 = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32)
+    o2, f2 = ops._fused_chunk_state_state_passing_fwd(Bd, xd * 2, dtd, dAd, torch.float32)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, 2 * o1) and torch.equal(f2, 2 * f1)
+    assert (o1[:, 0] == 0).all()
+
+
+def test_non_default_stream(ops, oracle):
+    d = oracle.make_inputs(1, b=1, L=512, H=4)
+    Bd, xd, dtd, dAd = map(_dev, (d["B"], d["x"], d["dt"], d["dA_cumsum"]))
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        out, fin = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32)
+    s.synchronize()
+    wo, wf = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    _check("stream.out", out, wo)
+
+
+def test_reference_module_names_resolve(ops):
+    from kernels.ssd_chunk_state import _chunk_state_fwd
+    from kernels.ssd_state_passing import _state_passing_fwd
+    from kernels.fused_globalbar import _fused_chunk_state_state_passing_fwd_globalbar
+    from kernels.fused_concurrent import _fused_chunk_state_state_passing_fwd_concurrent
+    assert _chunk_state_fwd is ops._chunk_state_fwd and _state_passing_fwd is ops._state_passing_fwd
+    assert callable(_fused_chunk_state_state_passing_fwd_globalbar) and callable(_fused_chunk_state_state_passing_fwd_concurrent)
