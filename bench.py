@@ -18,6 +18,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
+# HBM bytes per fused launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB -> bytes; the
+# factors are what the same counters read for a plain 1 GiB copy).  Keyed by workload name; see the rocprof summaries
+# kept with the repository.  None = not measured for that workload / kernel version.
+MEASURED_TRAFFIC_BYTES = {"cfg2_mamba2_2p7b": None}
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 
 
@@ -34,6 +38,9 @@ def main():
     ap.add_argument("--sets", type=int, default=3, help="rotating input/output buffer sets (defeats cache reuse)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--with-states", action="store_true", help="also materialise the per-chunk states")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 1 GiB device copy three times (the known-size kernel that the FETCH_SIZE / "
+                         "WRITE_SIZE counters are scaled by) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU only (the driver's boxes have one GPU, and the path needs "
@@ -48,6 +55,14 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        a = torch.ones(1 << 28, dtype=torch.float32, device=dev)      # 1 GiB
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": "3 x copy of 1073741824 bytes (1048576 KiB read, 1048576 KiB written each)"}))
+        return
     cfg = ssd_oracle.CONFIGS[args.config]
     log(f"[bench] workload {cfg['name']}: {cfg}")
     d = ssd_oracle.make_inputs(args.config)
@@ -121,7 +136,8 @@ def main():
                                f"{cfg['dtype']} x/B, fp32 dt/dA_cumsum/out/final",
                    "materialise_states": bool(args.with_states), "buffer_sets": nsets},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None if args.with_states else MEASURED_TRAFFIC_BYTES.get(cfg["name"]),
                      "algorithmic_bytes": alg_bytes, "kernel_us": round(ev_step * 1e6, 2)},
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
