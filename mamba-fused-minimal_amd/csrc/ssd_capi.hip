@@ -22,7 +22,6 @@ int check_device()
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return SSD_ERR_DEVICE;
     const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-    if (const char *e = getenv("SSD_PREFETCH_WAVE")) ssd::set_prefetch_wave(atoi(e));
     if (dev < 64) cached[dev] = ok ? 1 : 2;
     return ok ? SSD_OK : SSD_ERR_DEVICE;
 }

@@ -46,12 +46,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// Workgroup barrier that only orders LDS traffic (global loads issued earlier stay in flight).
+// Workgroup barrier that only orders the LDS reads and writes made by ds instructions: global loads issued
+// earlier -- including the ones that deposit x rows in LDS, which a release fence would wait for -- stay in
+// flight.  s_waitcnt lgkmcnt(0) (vmcnt and expcnt fields left at their maxima) completes this wave's ds
+// operations; the barrier intrinsic keeps the compiler from moving memory operations across it.
 __device__ __forceinline__ void lds_barrier()
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // Store HB consecutive state values of one row (fp32, bf16 or f16 destination) with a raw buffer store:
@@ -124,24 +126,29 @@ __device__ __forceinline__ void exchange_read(const f32x4 (&acc)[2][NB], const f
                                               float (&sum)[2][NB])
 {
     constexpr int NU = NB / 4;
+    f32x4 part[3][2][NU];               // all reads in flight before the first add
+#pragma unroll
+    for (int r = 1; r < 4; ++r)
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+            for (int u = 0; u < NU; ++u) part[r - 1][jp][u] = red[(((wave * 3 + (r - 1)) * 2 + jp) * NU + u) * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int jp = 0; jp < 2; ++jp)
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             f32x4 t = {acc[jp][4 * u][0], acc[jp][4 * u + 1][0], acc[jp][4 * u + 2][0], acc[jp][4 * u + 3][0]};
 #pragma unroll
-            for (int r = 1; r < 4; ++r)         // fixed order: own quarter, then the three others
-                t += red[(((wave * 3 + (r - 1)) * 2 + jp) * NU + u) * 64 + lane];
+            for (int r = 1; r < 4; ++r) t += part[r - 1][jp][u];   // fixed order: own quarter, then the three others
             sum[jp][4 * u] = t.x; sum[jp][4 * u + 1] = t.y; sum[jp][4 * u + 2] = t.z; sum[jp][4 * u + 3] = t.w;
         }
 }
 
-constexpr int kXPitch = 72;      // bytes per staged x row in LDS (64 data + 8 pad: conflict-free operand reads)
-
 template <int NB, int KS> constexpr int lds_bytes()
 {
     return 12 * 2 * (NB / 4) * 64 * 16      // token-split exchange
-           + 4 * 32 * KS * kXPitch          // x staging, one area per wave
+           + 4 * 32 * KS * 64               // x rows, one area per wave
            + 4 * 32 * KS * 4;               // per-token weights
 }
 
@@ -153,13 +160,13 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     constexpr int NBD = NB / 2;         // dwords of B per lane per row
     constexpr int NU = NB / 4;          // 128-bit units per state row per lane
     constexpr int QW = 32 * KS;         // tokens per wave per chunk
-    constexpr int NXW = QW / 16;        // 16-byte x loads per lane per chunk
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
-    f32x4 *red = (f32x4 *)lds_raw;                                   // [(dst*3+slot)*2+jp][u][lane]
-    char *xst_all = lds_raw + 12 * 2 * NU * 64 * 16;
-    float *wbuf = (float *)(xst_all + 4 * QW * kXPitch);
+    char *xst_all = lds_raw;                                          // x rows: the first 8 or 16 KB
+    float *wbuf = (float *)(xst_all + 4 * QW * 64);
+    f32x4 *red = (f32x4 *)(xst_all + 4 * QW * 68);                    // [(dst*3+slot)*2+jp][u][lane]
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i16 = lane & 15, kg = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, kg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     // Work item -> (batch, [chunk,] head, row slice).  Consecutive items share B (same batch, same group) and
     // are placed on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so that B tiles and the
@@ -204,33 +211,41 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
 
     // B: lane (i16, kg) reads NB consecutive columns of the 8 tokens 8kg..8kg+7 of a step
     const int Blane = (int)((wave * QW + 8 * kg) * Brb) + 2 * NB * i16;
-    auto load_B = [&](int gstep, uint32_t (&bo)[8][NBD]) {       // gstep = (c - c_begin) * KS + s
+    auto load_B_row = [&](int gstep, int j, uint32_t (&bo)[NBD]) {      // gstep = (c - c_begin) * KS + s
         const int c = c_begin + gstep / KS, s = gstep % KS;
         const auto rs = chunk_rsrc(Brow, Brb, c);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if constexpr (NBD == 4) {
-                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, Blane, (int)((32 * s + j) * Brb), 0);
-                bo[j][0] = v.x; bo[j][1] = v.y; bo[j][2] = v.z; bo[j][3] = v.w;
-            } else {
-                const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, Blane, (int)((32 * s + j) * Brb), 0);
-                bo[j][0] = v.x; bo[j][1] = v.y;
-            }
+        if constexpr (NBD == 4) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, Blane, (int)((32 * s + j) * Brb), 0);
+            bo[0] = v.x; bo[1] = v.y; bo[2] = v.z; bo[3] = v.w;
+        } else {
+            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, Blane, (int)((32 * s + j) * Brb), 0);
+            bo[0] = v.x; bo[1] = v.y;
         }
     };
-    // x: 4 lanes per token row of the slice (16 bytes each), 16 token rows per instruction
-    const int xlane = (int)((wave * QW + (lane >> 2)) * xrb) + 2 * p0 + 16 * (lane & 3);
-    auto load_x = [&](int c, u32x4 (&xo)[NXW]) {
-        const auto rs = chunk_rsrc(xrow, xrb, c);
+    auto load_B = [&](int gstep, uint32_t (&bo)[8][NBD]) {
 #pragma unroll
-        for (int i = 0; i < NXW; ++i) xo[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, xlane, (int)(16 * i * xrb), 0);
+        for (int j = 0; j < 8; ++j) load_B_row(gstep, j, bo[j]);
     };
-    // LDS staging of this wave's x rows: written row-major, read back as (token, headdim row pair) dwords.
+    // x goes from global memory straight into a wave-private LDS area (buffer load with LDS destination:
+    // lane l deposits its 16 bytes at byte 16*l of a 1 KB block).  Two instructions cover the 32 token rows of a
+    // step; 4 lanes fetch one 64-byte row of the slice.  Which row a lane fetches is chosen so that the operand
+    // reads below are free of bank conflicts: instruction i puts token 8*kg + 4*i + m of the step at row slot
+    // 4*m + kg, so the four kg groups of a read hit four different 64-byte bank groups.
     // MFMA row i of this wave is headdim row pair rot(i) = 4*(i/4) + (i%4 + wave)%4 (see exchange_write).
-    char *xst = xst_all + wave * QW * kXPitch;
+    char *xst = xst_all + wave * QW * 64;
+    const int xlane = (int)((wave * QW + 8 * ((lane >> 2) & 3) + (lane >> 4)) * xrb) + 2 * p0 + 16 * (lane & 3);
+    auto load_x = [&](int c, int s, int i) {     // tokens 8*kg + 4*i + (0..3) of step s of chunk c
+        const auto rs = chunk_rsrc(xrow, xrb, c);
+#if defined(__HIP_DEVICE_COMPILE__)      // the LDS address space does not exist in the host pass
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xst + (2 * s + i) * 1024), 16, xlane,
+                                                 (int)((32 * s + 4 * i) * xrb), 0, 0);
+#else
+        (void)rs; (void)s; (void)i;
+#endif
+    };
     const int rot = (i16 & ~3) | ((i16 + wave) & 3);
-    const int xst_wr = (lane >> 2) * kXPitch + 16 * (lane & 3);
-    const int xst_rd = 8 * kg * kXPitch + 4 * rot;
+    const int xst_rd = 64 * kg + 4 * rot;         // + 1024 * (2*s + j/4) + 256 * (j%4) for token j of step s
 
     // Per-chunk scalars and per-token decay inputs, fetched one chunk ahead of their use.
     struct Meta { float dtv, cs, last; int32_t id, id_last; };
@@ -248,10 +263,17 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
         return m;
     };
 
-    u32x4 xw[NXW];
     uint32_t bX[8][NBD], bY[8][NBD], bZ[8][NBD];
     Meta mcur = load_meta(c_begin), mnext = mcur;
-    load_x(c_begin, xw);
+    // Rows past the end of the sequence are not fetched and may leave their LDS slots untouched; their weight
+    // is zero, so the slots only have to hold finite numbers.
+#pragma unroll
+    for (int i = 0; i < 2 * KS; ++i) *(u32x4 *)(xst + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): the zeros are in place before any row lands
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s = 0; s < KS; ++s) { load_x(c_begin, s, 0); load_x(c_begin, s, 1); }
+    __builtin_amdgcn_sched_barrier(0);           // the 16 B row loads below stay behind the x requests
     load_B(0, bX);
     load_B(1, bY);
 
@@ -290,22 +312,28 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
 #pragma unroll
                 for (int j = 0; j < NB; ++j) st[jp][j] = 0.f;
             }
-            // out[:, 0] = initial state (kernels/ssd_state_passing.py:66)
-            store_tile_row(slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + h * p.so_h, slice_out), dt_out, vo_out,
-                           jp * (int)p.so_p, st[jp]);
         }
     }
     int32_t prev_id = 0;
     int gstep = 0;
 
-    // One 32-token step of this wave: bc holds the step's raw B rows, bn receives those of two steps ahead.
-    auto step = [&](int s, f32x4 (&acc)[2][NB], uint32_t (&bc)[8][NBD], uint32_t (&bn)[8][NBD]) {
-        load_B(gstep + 2, bn);
-        __builtin_amdgcn_sched_barrier(0);       // keep the prefetch ahead of this step's waits
-
+    // One 32-token step of this wave of chunk c: bc holds the step's raw B rows, bn receives those of two steps
+    // ahead.  All memory instructions of the step -- the B rows for step + 2, the x rows of the same step of the
+    // next chunk, the state entering this chunk (out[:, c], kernels/ssd_state_passing.py:66-84) and the
+    // next chunk's decay inputs -- are spread over the MFMA loop, one or two per four MFMAs: a burst of them
+    // would stall the wave on the memory pipeline's issue queue.
+    auto step = [&](int c, int s, f32x4 (&acc)[2][NB], uint32_t (&bc)[8][NBD], uint32_t (&bn)[8][NBD]) {
+        // The x rows of this step were requested one chunk ago, as the first two vector-memory operations of
+        // the same step (or in the prologue, before 16 B rows).  Memory operations complete in order, so the rows
+        // are in LDS once no more than the operations issued after them are outstanding: at least the B rows of
+        // the rest of that step and 8 B rows + 2 x requests for every other step of the chunk.  The compiler does
+        // not track this dependence; the wait is explicit.
+        constexpr int kAfterX = (8 - 2 * (8 / NB)) + (KS - 1) * 10;
+        __builtin_amdgcn_s_waitcnt((kAfterX & 15) | (7 << 4) | (15 << 8) | ((kAfterX >> 4) << 14));
         uint32_t xr[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) xr[j] = *(const uint32_t *)(xst + xst_rd + (32 * s + j) * kXPitch);
+        for (int j = 0; j < 8; ++j)
+            xr[j] = *(const uint32_t *)(xst + xst_rd + 1024 * (2 * s + (j >> 2)) + 256 * (j & 3));
         const f32x4 wlo = *(const f32x4 *)&wbuf[wave * QW + 32 * s + 8 * kg];
         const f32x4 whi = *(const f32x4 *)&wbuf[wave * QW + 32 * s + 8 * kg + 4];
         const float wv[8] = {wlo.x, wlo.y, wlo.z, wlo.w, whi.x, whi.y, whi.z, whi.w};
@@ -331,6 +359,9 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
             Ahi[jp] = __builtin_bit_cast(bf16x8, (u32x4){ahi[jp][0], ahi[jp][1], ahi[jp][2], ahi[jp][3]});
             Alo[jp] = __builtin_bit_cast(bf16x8, (u32x4){alo[jp][0], alo[jp][1], alo[jp][2], alo[jp][3]});
         }
+        // Everything that reads this step's x rows is complete above this line; the requests that overwrite
+        // them with the next chunk's rows are issued below it.
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jn = 0; jn < NB; ++jn) {
             const uint32_t sel = (jn & 1) ? 0x07060302u : 0x05040100u;
@@ -345,6 +376,17 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
                 acc[jp][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ahi[jp], Bf, acc[jp][jn], 0, 0, 0);
                 acc[jp][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Alo[jp], Bf, acc[jp][jn], 0, 0, 0);
             }
+#pragma unroll
+            for (int j = jn * 8 / NB; j < (jn + 1) * 8 / NB; ++j) load_B_row(gstep + 2, j, bn[j]);
+            if (jn < 2) load_x(c + 1, s, jn);
+            if (FUSED && s == 0 && jn >= 2 && jn < 2 + 2 * NU) {
+                const int jp = (jn - 2) / NU, u = (jn - 2) % NU;
+                const float q[4] = {st[jp][4 * u], st[jp][4 * u + 1], st[jp][4 * u + 2], st[jp][4 * u + 3]};
+                store_row<4>(slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + c * p.so_c + h * p.so_h, slice_out), dt_out,
+                             vo_out, jp * (int)p.so_p + 4 * u, q);
+            }
+            if (s == 0 && jn == NB - 1) mnext = load_meta(min(c + 1, c_end - 1));
+            __builtin_amdgcn_sched_barrier(0);
         }
         ++gstep;
     };
@@ -352,8 +394,6 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     // One chunk.  b0 (and b1 when KS == 2) hold the raw B rows of its steps; three buffers rotate so that every
     // step can prefetch two steps ahead.
     auto chunk = [&](int c, uint32_t (&b0)[8][NBD], uint32_t (&b1)[8][NBD], uint32_t (&b2)[8][NBD]) {
-        mnext = load_meta(min(c + 1, c_end - 1));
-
         // ---- per-token weights of this wave's token quarter (kernels/ssd_chunk_state.py:134-156)
         {
             float e = mcur.last - mcur.cs;
@@ -363,16 +403,9 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
             if (HAS_SEQ && mcur.id != mcur.id_last) wv = 0.f;
             wbuf[wave * QW + (lane & (QW - 1))] = wv;
         }
-        // ---- stage this wave's x rows (fetched during the previous chunk), then fetch the next chunk's
-#pragma unroll
-        for (int i = 0; i < NXW; ++i) {
-            *(u32x2 *)(xst + xst_wr + 16 * i * kXPitch) = (u32x2){xw[i].x, xw[i].y};
-            *(u32x2 *)(xst + xst_wr + 16 * i * kXPitch + 8) = (u32x2){xw[i].z, xw[i].w};
-        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        load_x(c + 1, xw);
 
         f32x4 acc[2][NB];
 #pragma unroll
@@ -381,10 +414,10 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
             for (int jn = 0; jn < NB; ++jn) acc[jp][jn] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
         if constexpr (KS == 2) {
-            step(0, acc, b0, b2);
-            step(1, acc, b1, b0);
+            step(c, 0, acc, b0, b2);
+            step(c, 1, acc, b1, b0);
         } else {
-            step(0, acc, b0, b2);
+            step(c, 0, acc, b0, b2);
         }
 
         // ---- sum the four token quarters
@@ -410,12 +443,6 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
             for (int jp = 0; jp < 2; ++jp) {
 #pragma unroll
                 for (int j = 0; j < NB; ++j) st[jp][j] = sc * st[jp][j] + sum[jp][j];
-                if (c < p.C - 1)
-                    store_tile_row(slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + (c + 1) * p.so_c + h * p.so_h, slice_out),
-                                   dt_out, vo_out, jp * (int)p.so_p, st[jp]);
-                else
-                    store_tile_row(slice_rsrc(p.fin, 4, b * p.sf_b + h * p.sf_h, slice_fin), DT_F32, vo_fin,
-                                   jp * (int)p.sf_p, st[jp]);
             }
         }
         mcur = mnext;
@@ -434,6 +461,12 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
             chunk(c, bY, bZ, bX); if (++c >= c_end) break;
             chunk(c, bZ, bX, bY); if (++c >= c_end) break;
         }
+    }
+    if (FUSED) {
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp)
+            store_tile_row(slice_rsrc(p.fin, 4, b * p.sf_b + h * p.sf_h, slice_fin), DT_F32, vo_fin, jp * (int)p.sf_p,
+                           st[jp]);
     }
 }
 
@@ -460,8 +493,6 @@ bool mfma_supported(const Params &p)
     if (!ok16(p.init, p.sin_b, p.sin_h, p.sin_p, 0)) return false;
     return true;
 }
-
-void set_prefetch_wave(int) {}
 
 template <int NB, int KS, bool SEQ, bool FUSED>
 static hipError_t launch_one(const Params &p, dim3 grid, hipStream_t s)

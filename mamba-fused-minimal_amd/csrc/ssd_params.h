@@ -78,6 +78,5 @@ hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
-void set_prefetch_wave(int on);
 
 }  // namespace ssd
