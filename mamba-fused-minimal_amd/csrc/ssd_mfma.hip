@@ -58,6 +58,9 @@ __device__ __forceinline__ void lds_barrier()
 
 // Store HB consecutive state values of one row (fp32, bf16 or f16 destination) with a raw buffer store:
 // scalar descriptor + scalar element offset `soff` + loop-invariant per-lane element offset `voff`.
+// The data registers of a wide store are read out over several cycles after issue; when the compiler reuses the
+// register tuple for the next store and writes it in the very next instruction, some lanes were seen to store the
+// new value.  Each store is therefore followed by wait states that depend on its data registers.
 template <int HB>
 __device__ __forceinline__ void store_row(__amdgpu_buffer_rsrc_t rs, int dt, int voff, int soff, const float (&v)[HB])
 {
@@ -66,9 +69,11 @@ __device__ __forceinline__ void store_row(__amdgpu_buffer_rsrc_t rs, int dt, int
             const u32x4 q = {__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
                              __builtin_bit_cast(uint32_t, v[2]), __builtin_bit_cast(uint32_t, v[3])};
             __builtin_amdgcn_raw_buffer_store_b128(q, rs, 4 * voff, 4 * soff, 0);
+            asm volatile("s_nop 3" ::"v"(q) : "memory");
         } else {
             const u32x2 q = {__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1])};
             __builtin_amdgcn_raw_buffer_store_b64(q, rs, 4 * voff, 4 * soff, 0);
+            asm volatile("s_nop 3" ::"v"(q) : "memory");
         }
     } else {
         uint32_t w[HB / 2];
@@ -85,6 +90,7 @@ __device__ __forceinline__ void store_row(__amdgpu_buffer_rsrc_t rs, int dt, int
         if constexpr (HB == 4) {
             const u32x2 q = {w[0], w[1]};
             __builtin_amdgcn_raw_buffer_store_b64(q, rs, 2 * voff, 2 * soff, 0);
+            asm volatile("s_nop 3" ::"v"(q) : "memory");
         } else {
             __builtin_amdgcn_raw_buffer_store_b32(w[0], rs, 2 * voff, 2 * soff, 0);
         }
@@ -241,7 +247,7 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xst + (2 * s + i) * 1024), 16, xlane,
                                                  (int)((32 * s + 4 * i) * xrb), 0, 0);
 #else
-        (void)rs; (void)s; (void)i;
+        (void)rs; (void)s; (void)i; (void)xlane;
 #endif
     };
     const int rot = (i16 & ~3) | ((i16 + wave) & 3);
