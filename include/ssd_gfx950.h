@@ -116,6 +116,14 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  */
 int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
 
+/*
+ * Tuning / test hook with no counterpart in the reference: how many waves split the tokens of a chunk in the bf16
+ * MFMA kernels.  0 = let the library choose from the problem size (the default), 2 or 4 = force that split for
+ * every later call of this process.  Returns the previous setting, or SSD_ERR_SHAPE for any other value.
+ * Results agree between the settings to rounding (the tokens are summed in another order), not bit for bit.
+ */
+int ssd_set_token_split(int waves);
+
 #ifdef __cplusplus
 }
 #endif

@@ -186,4 +186,10 @@ int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dim
     return ssd::mfma_supported(p) ? 1 : 0;
 }
 
+int ssd_set_token_split(int waves)
+{
+    if (waves != 0 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;
+    return ssd::set_token_split(waves);
+}
+
 }  // extern "C"

@@ -107,69 +107,83 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t slice_rsrc(void *base, int esi
 
 __device__ __forceinline__ int esize_of(int dt) { return dt == DT_F32 ? 4 : 2; }
 
-// Token-split reduction through LDS.  Every wave rotates the headdim rows it feeds to the MFMA (see `rot` in the
-// kernel) so that accumulator component r of wave w holds rows owned by wave (w + r) % 4: component 0 stays,
-// components 1..3 go to the three other waves.  The code is the same for all waves; only addresses differ.
-template <int NB>
+// Token-split reduction through LDS.  WV waves split the tokens of a chunk.  Every wave rotates the headdim rows it
+// feeds to the MFMA (see `rot` in the kernel) so that accumulator component r = q*WV + d of wave w holds rows owned
+// by wave (w + d) % WV: components with d == 0 stay, the others go to the WV-1 other waves, where they add to that
+// wave's component q*WV.  The code is the same for all waves; only addresses differ.
+// Layout of `red`: [destination wave][d-1][q][jp][unit][lane] of 16-byte units.
+template <int NB, int WV>
 __device__ __forceinline__ void exchange_write(const f32x4 (&acc)[2][NB], f32x4 *red, int wave, int lane)
 {
-    constexpr int NU = NB / 4;
+    constexpr int NU = NB / 4, NOWN = 4 / WV;
 #pragma unroll
-    for (int r = 1; r < 4; ++r) {
-        const int dst = (wave + r) & 3;
+    for (int d = 1; d < WV; ++d) {
+        const int dst = (wave + d) & (WV - 1);
+#pragma unroll
+        for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    const int r = q * WV + d;
+                    const f32x4 v = {acc[jp][4 * u][r], acc[jp][4 * u + 1][r], acc[jp][4 * u + 2][r], acc[jp][4 * u + 3][r]};
+                    red[((((dst * (WV - 1) + (d - 1)) * NOWN + q) * 2 + jp) * NU + u) * 64 + lane] = v;
+                }
+    }
+}
+
+template <int NB, int WV>
+__device__ __forceinline__ void exchange_read(const f32x4 (&acc)[2][NB], const f32x4 *red, int wave, int lane,
+                                              float (&sum)[4 / WV][2][NB])
+{
+    constexpr int NU = NB / 4, NOWN = 4 / WV;
+    f32x4 part[WV - 1][NOWN][2][NU];    // all reads in flight before the first add
+#pragma unroll
+    for (int d = 1; d < WV; ++d)
+#pragma unroll
+        for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+                for (int u = 0; u < NU; ++u)
+                    part[d - 1][q][jp][u] = red[((((wave * (WV - 1) + (d - 1)) * NOWN + q) * 2 + jp) * NU + u) * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < NOWN; ++q)
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp)
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
-                const f32x4 v = {acc[jp][4 * u][r], acc[jp][4 * u + 1][r], acc[jp][4 * u + 2][r], acc[jp][4 * u + 3][r]};
-                red[(((dst * 3 + (r - 1)) * 2 + jp) * NU + u) * 64 + lane] = v;
+                const int r = q * WV;
+                f32x4 t = {acc[jp][4 * u][r], acc[jp][4 * u + 1][r], acc[jp][4 * u + 2][r], acc[jp][4 * u + 3][r]};
+#pragma unroll
+                for (int d = 1; d < WV; ++d) t += part[d - 1][q][jp][u];   // fixed order: own part, then the others
+                sum[q][jp][4 * u] = t.x; sum[q][jp][4 * u + 1] = t.y; sum[q][jp][4 * u + 2] = t.z; sum[q][jp][4 * u + 3] = t.w;
             }
-    }
 }
 
-template <int NB>
-__device__ __forceinline__ void exchange_read(const f32x4 (&acc)[2][NB], const f32x4 *red, int wave, int lane,
-                                              float (&sum)[2][NB])
+template <int NB, int KS, int WV> constexpr int lds_bytes()
 {
-    constexpr int NU = NB / 4;
-    f32x4 part[3][2][NU];               // all reads in flight before the first add
-#pragma unroll
-    for (int r = 1; r < 4; ++r)
-#pragma unroll
-        for (int jp = 0; jp < 2; ++jp)
-#pragma unroll
-            for (int u = 0; u < NU; ++u) part[r - 1][jp][u] = red[(((wave * 3 + (r - 1)) * 2 + jp) * NU + u) * 64 + lane];
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int jp = 0; jp < 2; ++jp)
-#pragma unroll
-        for (int u = 0; u < NU; ++u) {
-            f32x4 t = {acc[jp][4 * u][0], acc[jp][4 * u + 1][0], acc[jp][4 * u + 2][0], acc[jp][4 * u + 3][0]};
-#pragma unroll
-            for (int r = 1; r < 4; ++r) t += part[r - 1][jp][u];   // fixed order: own quarter, then the three others
-            sum[jp][4 * u] = t.x; sum[jp][4 * u + 1] = t.y; sum[jp][4 * u + 2] = t.z; sum[jp][4 * u + 3] = t.w;
-        }
+    return WV * (WV - 1) * (4 / WV) * 2 * (NB / 4) * 64 * 16      // token-split exchange
+           + WV * 32 * KS * 64                                    // x rows, one area per wave
+           + WV * 32 * KS * 4;                                    // per-token weights
 }
 
-template <int NB, int KS> constexpr int lds_bytes()
-{
-    return 12 * 2 * (NB / 4) * 64 * 16      // token-split exchange
-           + 4 * 32 * KS * 64               // x rows, one area per wave
-           + 4 * 32 * KS * 4;               // per-token weights
-}
-
-// NB = dstate / 16 (4 or 8); KS = 32-token steps per wave per chunk (chunk_size = 128 * KS);
-// ALL32 = initial states, states, out are all fp32 (or absent): element-type branches fold away.
-template <int NB, int KS, bool HAS_SEQ, bool FUSED, bool ALL32>
-__global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
+// NB = dstate / 16 (4 or 8); WV = waves per workgroup = token split (2 or 4); KS = 32-token steps per wave per
+// chunk (chunk_size = 32 * KS * WV); ALL32 = initial states, states, out are all fp32 (or absent): element-type
+// branches fold away.
+template <int NB, int KS, int WV, bool HAS_SEQ, bool FUSED, bool ALL32>
+__global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
 {
     constexpr int NBD = NB / 2;         // dwords of B per lane per row
     constexpr int NU = NB / 4;          // 128-bit units per state row per lane
     constexpr int QW = 32 * KS;         // tokens per wave per chunk
+    constexpr int NOWN = 4 / WV;        // accumulator components (MFMA row groups) a wave owns after the reduction
+    constexpr int TPL = QW > 64 ? QW / 64 : 1;      // tokens per lane when the wave's weights are computed
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     char *xst_all = lds_raw;                                          // x rows: the first 8 or 16 KB
-    float *wbuf = (float *)(xst_all + 4 * QW * 64);
-    f32x4 *red = (f32x4 *)(xst_all + 4 * QW * 68);                    // [(dst*3+slot)*2+jp][u][lane]
+    float *wbuf = (float *)(xst_all + WV * QW * 64);
+    f32x4 *red = (f32x4 *)(xst_all + WV * QW * 68);
 
     const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, kg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -237,7 +251,7 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     // step; 4 lanes fetch one 64-byte row of the slice.  Which row a lane fetches is chosen so that the operand
     // reads below are free of bank conflicts: instruction i puts token 8*kg + 4*i + m of the step at row slot
     // 4*m + kg, so the four kg groups of a read hit four different 64-byte bank groups.
-    // MFMA row i of this wave is headdim row pair rot(i) = 4*(i/4) + (i%4 + wave)%4 (see exchange_write).
+    // MFMA row i of this wave is headdim row pair rot(i) = WV*(i/WV) + (i%WV + wave)%WV (see exchange_write).
     char *xst = xst_all + wave * QW * 64;
     const int xlane = (int)((wave * QW + 8 * ((lane >> 2) & 3) + (lane >> 4)) * xrb) + 2 * p0 + 16 * (lane & 3);
     auto load_x = [&](int c, int s, int i) {     // tokens 8*kg + 4*i + (0..3) of step s of chunk c
@@ -250,20 +264,26 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
         (void)rs; (void)s; (void)i; (void)xlane;
 #endif
     };
-    const int rot = (i16 & ~3) | ((i16 + wave) & 3);
+    const int rot = (i16 & ~(WV - 1)) | ((i16 + wave) & (WV - 1));
     const int xst_rd = 64 * kg + 4 * rot;         // + 1024 * (2*s + j/4) + 256 * (j%4) for token j of step s
 
     // Per-chunk scalars and per-token decay inputs, fetched one chunk ahead of their use.
-    struct Meta { float dtv, cs, last; int32_t id, id_last; };
+    // Lane l looks after tokens TPL*l .. TPL*l + TPL-1 of the wave's share (lanes repeat when the share is < 64).
+    struct Meta { float dtv[TPL], cs[TPL], last; int32_t id[TPL], id_last; };
+    const int ktok = wave * QW + ((lane * TPL) & (QW - 1));
     auto load_meta = [&](int c) {
         Meta m;
-        const int k = wave * QW + (lane & (QW - 1));
-        m.dtv = dtb[c * p.sdt_c + k * p.sdt_k];
-        m.cs = dab[c * p.sda_c + k * p.sda_k];
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) {
+            m.dtv[t] = dtb[c * p.sdt_c + (ktok + t) * p.sdt_k];
+            m.cs[t] = dab[c * p.sda_c + (ktok + t) * p.sda_k];
+            m.id[t] = 0;
+        }
         m.last = dab[c * p.sda_c + (int64_t)(Q - 1) * p.sda_k];
-        m.id = 0; m.id_last = 0;
+        m.id_last = 0;
         if (HAS_SEQ) {
-            m.id = sqb[(int64_t)min(c * Q + k, L - 1) * p.ssq_l];
+#pragma unroll
+            for (int t = 0; t < TPL; ++t) m.id[t] = sqb[(int64_t)min(c * Q + ktok + t, L - 1) * p.ssq_l];
             m.id_last = sqb[(int64_t)(min((c + 1) * Q, L) - 1) * p.ssq_l];
         }
         return m;
@@ -282,8 +302,10 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     __builtin_amdgcn_sched_barrier(0);           // the 16 B row loads below stay behind the x requests
     load_B(0, bX);
     load_B(1, bY);
+    __builtin_amdgcn_s_waitcnt((16 & 15) | (7 << 4) | (15 << 8) | ((16 >> 4) << 14));   // vmcnt(16): x rows are in
 
-    // owner rows of this lane after the token reduction; element offsets inside one (headdim x dstate) slice
+    // Owner rows of this lane after the token reduction: owned component q covers headdim rows prow + 2*WV*q + jp.
+    // Element offsets inside one (headdim x dstate) slice.
     const int prow = p0 + 2 * (4 * kg + wave);
     const int ncol = NB * i16;
     const int vo_out = prow * (int)p.so_p + ncol, vo_st = prow * (int)p.sst_p + ncol, vo_fin = prow * (int)p.sf_p + ncol;
@@ -298,25 +320,27 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
         }
     };
 
-    float st[2][NB];
+    float st[NOWN][2][NB];
     if (FUSED) {
+#pragma unroll
+        for (int q = 0; q < NOWN; ++q)
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp) {
             if (p.init) {
-                const int64_t off = b * p.sin_b + h * p.sin_h + (int64_t)(prow + jp) * p.sin_p + ncol;
+                const int64_t off = b * p.sin_b + h * p.sin_h + (int64_t)(prow + 2 * WV * q + jp) * p.sin_p + ncol;
                 if (dt_init == DT_F32) {
 #pragma unroll
                     for (int u = 0; u < NU; ++u) {
-                        const f32x4 q = *(const f32x4 *)((const float *)p.init + off + 4 * u);
-                        st[jp][4 * u] = q.x; st[jp][4 * u + 1] = q.y; st[jp][4 * u + 2] = q.z; st[jp][4 * u + 3] = q.w;
+                        const f32x4 v = *(const f32x4 *)((const float *)p.init + off + 4 * u);
+                        st[q][jp][4 * u] = v.x; st[q][jp][4 * u + 1] = v.y; st[q][jp][4 * u + 2] = v.z; st[q][jp][4 * u + 3] = v.w;
                     }
                 } else {
 #pragma unroll
-                    for (int j = 0; j < NB; ++j) st[jp][j] = load_as_f32(p.init, off + j, dt_init);
+                    for (int j = 0; j < NB; ++j) st[q][jp][j] = load_as_f32(p.init, off + j, dt_init);
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < NB; ++j) st[jp][j] = 0.f;
+                for (int j = 0; j < NB; ++j) st[q][jp][j] = 0.f;
             }
         }
     }
@@ -385,11 +409,11 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
 #pragma unroll
             for (int j = jn * 8 / NB; j < (jn + 1) * 8 / NB; ++j) load_B_row(gstep + 2, j, bn[j]);
             if (jn < 2) load_x(c + 1, s, jn);
-            if (FUSED && s == 0 && jn >= 2 && jn < 2 + 2 * NU) {
-                const int jp = (jn - 2) / NU, u = (jn - 2) % NU;
-                const float q[4] = {st[jp][4 * u], st[jp][4 * u + 1], st[jp][4 * u + 2], st[jp][4 * u + 3]};
+            if (FUSED && s == 0 && jn < NOWN * 2 * NU) {      // NOWN * 2 * NU <= NB stores, one per iteration
+                const int q = jn / (2 * NU), jp = (jn / NU) % 2, u = jn % NU;
+                const float v[4] = {st[q][jp][4 * u], st[q][jp][4 * u + 1], st[q][jp][4 * u + 2], st[q][jp][4 * u + 3]};
                 store_row<4>(slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + c * p.so_c + h * p.so_h, slice_out), dt_out,
-                             vo_out, jp * (int)p.so_p + 4 * u, q);
+                             vo_out, (2 * WV * q + jp) * (int)p.so_p + 4 * u, v);
             }
             if (s == 0 && jn == NB - 1) mnext = load_meta(min(c + 1, c_end - 1));
             __builtin_amdgcn_sched_barrier(0);
@@ -401,13 +425,14 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     // step can prefetch two steps ahead.
     auto chunk = [&](int c, uint32_t (&b0)[8][NBD], uint32_t (&b1)[8][NBD], uint32_t (&b2)[8][NBD]) {
         // ---- per-token weights of this wave's token quarter (kernels/ssd_chunk_state.py:134-156)
-        {
-            float e = mcur.last - mcur.cs;
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) {
+            float e = mcur.last - mcur.cs[t];
             if (p.clamp) e = fminf(e, 0.f);
-            float wv = __expf(e) * mcur.dtv;
-            if (c * Q + wave * QW + (lane & (QW - 1)) >= L) wv = 0.f;
-            if (HAS_SEQ && mcur.id != mcur.id_last) wv = 0.f;
-            wbuf[wave * QW + (lane & (QW - 1))] = wv;
+            float wv = __expf(e) * mcur.dtv[t];
+            if (c * Q + ktok + t >= L) wv = 0.f;
+            if (HAS_SEQ && mcur.id[t] != mcur.id_last) wv = 0.f;
+            wbuf[ktok + t] = wv;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
@@ -419,25 +444,28 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
 #pragma unroll
             for (int jn = 0; jn < NB; ++jn) acc[jp][jn] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-        if constexpr (KS == 2) {
-            step(c, 0, acc, b0, b2);
-            step(c, 1, acc, b1, b0);
-        } else {
-            step(c, 0, acc, b0, b2);
+        step(c, 0, acc, b0, b2);
+        if constexpr (KS >= 2) step(c, 1, acc, b1, b0);
+        if constexpr (KS == 4) {
+            step(c, 2, acc, b2, b1);
+            step(c, 3, acc, b0, b2);
         }
 
-        // ---- sum the four token quarters
+        // ---- sum the token shares of the WV waves
         lds_barrier();                      // previous chunk's exchange reads are done
-        exchange_write<NB>(acc, red, wave, lane);
+        exchange_write<NB, WV>(acc, red, wave, lane);
         lds_barrier();
-        float sum[2][NB];
-        exchange_read<NB>(acc, red, wave, lane, sum);
+        float sum[NOWN][2][NB];
+        exchange_read<NB, WV>(acc, red, wave, lane, sum);
 
         // ---- per-chunk states (side output) and the recurrence (kernels/ssd_state_passing.py:69-84)
         if (p.states) {
             const auto rs = slice_rsrc(p.states, esize_of(dt_states), b * p.sst_b + c * p.sst_c + h * p.sst_h, slice_st);
 #pragma unroll
-            for (int jp = 0; jp < 2; ++jp) store_tile_row(rs, dt_states, vo_st, jp * (int)p.sst_p, sum[jp]);
+            for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+                for (int jp = 0; jp < 2; ++jp)
+                    store_tile_row(rs, dt_states, vo_st, (2 * WV * q + jp) * (int)p.sst_p, sum[q][jp]);
         }
         if (FUSED) {
             float sc = __expf(mcur.last);
@@ -446,16 +474,17 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
                 prev_id = mcur.id_last;
             }
 #pragma unroll
-            for (int jp = 0; jp < 2; ++jp) {
+            for (int q = 0; q < NOWN; ++q)
 #pragma unroll
-                for (int j = 0; j < NB; ++j) st[jp][j] = sc * st[jp][j] + sum[jp][j];
-            }
+                for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) st[q][jp][j] = sc * st[q][jp][j] + sum[q][jp][j];
         }
         mcur = mnext;
     };
 
     int c = c_begin;
-    if constexpr (KS == 2) {
+    if constexpr (KS == 2) {             // two steps rotate the three buffers by two; one or four steps by one
         for (;;) {
             chunk(c, bX, bY, bZ); if (++c >= c_end) break;
             chunk(c, bZ, bX, bY); if (++c >= c_end) break;
@@ -470,9 +499,11 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const Params p)
     }
     if (FUSED) {
 #pragma unroll
-        for (int jp = 0; jp < 2; ++jp)
-            store_tile_row(slice_rsrc(p.fin, 4, b * p.sf_b + h * p.sf_h, slice_fin), DT_F32, vo_fin, jp * (int)p.sf_p,
-                           st[jp]);
+        for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp)
+                store_tile_row(slice_rsrc(p.fin, 4, b * p.sf_b + h * p.sf_h, slice_fin), DT_F32, vo_fin,
+                               (2 * WV * q + jp) * (int)p.sf_p, st[q][jp]);
     }
 }
 
@@ -500,36 +531,39 @@ bool mfma_supported(const Params &p)
     return true;
 }
 
-template <int NB, int KS, bool SEQ, bool FUSED>
+template <int NB, int KS, int WV, bool SEQ, bool FUSED>
 static hipError_t launch_one(const Params &p, dim3 grid, hipStream_t s)
 {
     const bool all32 = (!p.out || p.dt_out == DT_F32) && (!p.states || p.dt_states == DT_F32) &&
                        (!p.init || p.dt_init == DT_F32);
-    constexpr int lds = lds_bytes<NB, KS>();
+    constexpr int lds = lds_bytes<NB, KS, WV>();
     // more than 64 KB of LDS per workgroup has to be requested explicitly, once per kernel
     static bool configured[2] = {false, false};
     if (lds > 65536 && !configured[all32]) {
-        hipError_t e = all32 ? hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, SEQ, FUSED, true>,
+        hipError_t e = all32 ? hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, true>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds)
-                             : hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, SEQ, FUSED, false>,
+                             : hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, false>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         configured[all32] = true;
     }
-    if (all32) hipLaunchKernelGGL((mfma_kernel<NB, KS, SEQ, FUSED, true>), grid, dim3(256), lds, s, p);
-    else hipLaunchKernelGGL((mfma_kernel<NB, KS, SEQ, FUSED, false>), grid, dim3(256), lds, s, p);
+    if (all32) hipLaunchKernelGGL((mfma_kernel<NB, KS, WV, SEQ, FUSED, true>), grid, dim3(64 * WV), lds, s, p);
+    else hipLaunchKernelGGL((mfma_kernel<NB, KS, WV, SEQ, FUSED, false>), grid, dim3(64 * WV), lds, s, p);
     return hipGetLastError();
 }
 
-template <int NB, int KS>
+template <int NB, int KS, int WV>
 static hipError_t launch_nb_ks(const Params &p, bool fused, hipStream_t s)
 {
     const int per_xcd = (p.n_items + 7) / 8;
     const bool seq = p.seq != nullptr;
     dim3 grid(per_xcd * 8);
-    if (fused) return seq ? launch_one<NB, KS, true, true>(p, grid, s) : launch_one<NB, KS, false, true>(p, grid, s);
-    return seq ? launch_one<NB, KS, true, false>(p, grid, s) : launch_one<NB, KS, false, false>(p, grid, s);
+    if (fused) return seq ? launch_one<NB, KS, WV, true, true>(p, grid, s) : launch_one<NB, KS, WV, false, true>(p, grid, s);
+    return seq ? launch_one<NB, KS, WV, true, false>(p, grid, s) : launch_one<NB, KS, WV, false, false>(p, grid, s);
 }
+
+static int g_force_split = 0;       // 0 = choose from the problem size; 2 or 4 = forced
+int set_token_split(int wv) { const int old = g_force_split; g_force_split = wv; return old; }
 
 hipError_t launch_mfma(const Params &p_in, bool fused, hipStream_t s)
 {
@@ -537,11 +571,24 @@ hipError_t launch_mfma(const Params &p_in, bool fused, hipStream_t s)
     const int n_pt = p.headdim / 32;
     p.n_items = fused ? p.batch * p.nheads * n_pt : p.batch * p.C * p.nheads * n_pt;
     if (p.n_items <= 0) return hipSuccess;
-    const int nb = p.dstate / 16, ks = p.Q / 128;
-    if (nb == 8 && ks == 2) return launch_nb_ks<8, 2>(p, fused, s);
-    if (nb == 8 && ks == 1) return launch_nb_ks<8, 1>(p, fused, s);
-    if (nb == 4 && ks == 2) return launch_nb_ks<4, 2>(p, fused, s);
-    return launch_nb_ks<4, 1>(p, fused, s);
+    // Token split.  The kernels are bound by instruction issue, and two waves per state tile need 17 % fewer
+    // vector instructions per tile than four (half the reduction traffic): measured 11-18 % faster for the
+    // unfused launch, whose (batch, chunk, head, slice) items are plentiful.  The fused launch walks the chunks of
+    // a tile serially with the running state in registers; there four waves win (2-wave workgroups spill and a
+    // tile's chunk takes twice as long), 285 vs 361 us at b=4 L=8192 H=80.
+    int wv = (!fused && p.n_items > 512) ? 2 : 4;
+    if (g_force_split == 2 || g_force_split == 4) wv = g_force_split;
+    const int nb = p.dstate / 16, q128 = p.Q / 128;     // chunk 128 or 256
+    if (wv == 4) {
+        if (nb == 8 && q128 == 2) return launch_nb_ks<8, 2, 4>(p, fused, s);
+        if (nb == 8 && q128 == 1) return launch_nb_ks<8, 1, 4>(p, fused, s);
+        if (nb == 4 && q128 == 2) return launch_nb_ks<4, 2, 4>(p, fused, s);
+        return launch_nb_ks<4, 1, 4>(p, fused, s);
+    }
+    if (nb == 8 && q128 == 2) return launch_nb_ks<8, 4, 2>(p, fused, s);
+    if (nb == 8 && q128 == 1) return launch_nb_ks<8, 2, 2>(p, fused, s);
+    if (nb == 4 && q128 == 2) return launch_nb_ks<4, 4, 2>(p, fused, s);
+    return launch_nb_ks<4, 2, 2>(p, fused, s);
 }
 
 }  // namespace ssd

@@ -78,5 +78,6 @@ hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
+int set_token_split(int wv);      // 0 = automatic; 2 or 4 forces the token split of the MFMA kernels; returns the old value
 
 }  // namespace ssd

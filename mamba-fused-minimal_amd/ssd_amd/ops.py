@@ -150,3 +150,12 @@ def _fused_chunk_state_state_passing_fwd_concurrent(B, x, dt, dA_cumsum, out_dty
     """Drop-in for kernels/fused_concurrent.py:255 (same signature and returns; prints nothing)."""
     return _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=initial_states,
                                                 seq_idx=seq_idx, states=states, states_in_fp32=states_in_fp32)
+
+
+def set_token_split(waves):
+    """Tuning / test hook (no counterpart in the reference): force how many waves split the tokens of a chunk in
+    the bf16 MFMA kernels (2 or 4), or 0 to let the library choose.  Returns the previous setting."""
+    rc = _lib.load().ssd_set_token_split(int(waves))
+    if rc < 0:
+        raise ValueError("token split must be 0, 2 or 4")
+    return rc
