@@ -162,11 +162,19 @@ __device__ __forceinline__ void exchange_read(const f32x4 (&acc)[2][NB], const f
             }
 }
 
-template <int NB, int KS, int WV> constexpr int lds_bytes()
+// With two waves per tile the running state of the fused kernel lives in LDS (32 values per lane would not fit
+// the register file next to the accumulators and the three B buffers); with four waves it stays in registers (16
+// values per lane; the 16 KB would push the workgroup past half of the 160 KB of a compute unit).
+template <int WV> constexpr bool state_in_lds() { return WV == 2; }
+
+template <int NB, int WV> constexpr int exchange_bytes() { return WV * (WV - 1) * (4 / WV) * 2 * (NB / 4) * 64 * 16; }
+
+template <int NB, int KS, int WV, bool FUSED> constexpr int lds_bytes()
 {
-    return WV * (WV - 1) * (4 / WV) * 2 * (NB / 4) * 64 * 16      // token-split exchange
+    return exchange_bytes<NB, WV>()                               // token-split exchange
            + WV * 32 * KS * 64                                    // x rows, one area per wave
-           + WV * 32 * KS * 4;                                    // per-token weights
+           + WV * 32 * KS * 4                                     // per-token weights
+           + (FUSED && state_in_lds<WV>() ? 32 * NB * 16 * 4 : 0);   // running state of the tile
 }
 
 // NB = dstate / 16 (4 or 8); WV = waves per workgroup = token split (2 or 4); KS = 32-token steps per wave per
@@ -184,9 +192,12 @@ __global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
     char *xst_all = lds_raw;                                          // x rows: the first 8 or 16 KB
     float *wbuf = (float *)(xst_all + WV * QW * 64);
     f32x4 *red = (f32x4 *)(xst_all + WV * QW * 68);
+    constexpr bool ST_LDS = FUSED && state_in_lds<WV>();
 
     const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, kg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // running state in LDS: [wave][owned component q][jp][unit] of 64 lanes x 16 bytes, lane-private
+    f32x4 *stl = (f32x4 *)((char *)red + exchange_bytes<NB, WV>()) + wave * NOWN * 2 * NU * 64 + lane;
 
     // Work item -> (batch, [chunk,] head, row slice).  Consecutive items share B (same batch, same group) and
     // are placed on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so that B tiles and the
@@ -320,8 +331,26 @@ __global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
         }
     };
 
-    float st[NOWN][2][NB];
-    if (FUSED) {
+    float st[ST_LDS ? 1 : NOWN][2][NB];
+    if (ST_LDS) {
+        // out[:, 0] = initial state (kernels/ssd_state_passing.py:66), and the state's home in LDS
+        const auto rs0 = slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + c_begin * p.so_c + h * p.so_h, slice_out);
+#pragma unroll
+        for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    float v[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (p.init) {
+                        const int64_t off = b * p.sin_b + h * p.sin_h + (int64_t)(prow + 2 * WV * q + jp) * p.sin_p + ncol + 4 * u;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) v[j] = load_as_f32(p.init, off + j, dt_init);
+                    }
+                    stl[((q * 2 + jp) * NU + u) * 64] = (f32x4){v[0], v[1], v[2], v[3]};
+                    store_row<4>(rs0, dt_out, vo_out, (2 * WV * q + jp) * (int)p.so_p + 4 * u, v);
+                }
+    } else if (FUSED) {
 #pragma unroll
         for (int q = 0; q < NOWN; ++q)
 #pragma unroll
@@ -409,7 +438,7 @@ __global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
 #pragma unroll
             for (int j = jn * 8 / NB; j < (jn + 1) * 8 / NB; ++j) load_B_row(gstep + 2, j, bn[j]);
             if (jn < 2) load_x(c + 1, s, jn);
-            if (FUSED && s == 0 && jn < NOWN * 2 * NU) {      // NOWN * 2 * NU <= NB stores, one per iteration
+            if (FUSED && !ST_LDS && s == 0 && jn < NOWN * 2 * NU) {      // NOWN * 2 * NU <= NB stores, one per iteration
                 const int q = jn / (2 * NU), jp = (jn / NU) % 2, u = jn % NU;
                 const float v[4] = {st[q][jp][4 * u], st[q][jp][4 * u + 1], st[q][jp][4 * u + 2], st[q][jp][4 * u + 3]};
                 store_row<4>(slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + c * p.so_c + h * p.so_h, slice_out), dt_out,
@@ -473,12 +502,33 @@ __global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
                 if (mcur.id_last != prev_id) sc = 0.f;
                 prev_id = mcur.id_last;
             }
+            if constexpr (ST_LDS) {
+                // state <- sc * state + sum, back to LDS and out to out[:, c + 1] (or final_states after the last chunk)
+                const bool last = c == p.C - 1;
+                const auto rs = last ? slice_rsrc(p.fin, 4, b * p.sf_b + h * p.sf_h, slice_fin)
+                                     : slice_rsrc(p.out, esize_of(dt_out), b * p.so_b + (c + 1) * p.so_c + h * p.so_h, slice_out);
+                const int dt_dst = last ? (int)DT_F32 : dt_out;
+                const int vo = last ? vo_fin : vo_out, pitch = last ? (int)p.sf_p : (int)p.so_p;
 #pragma unroll
-            for (int q = 0; q < NOWN; ++q)
+                for (int q = 0; q < NOWN; ++q)
 #pragma unroll
-                for (int jp = 0; jp < 2; ++jp)
+                    for (int jp = 0; jp < 2; ++jp)
 #pragma unroll
-                    for (int j = 0; j < NB; ++j) st[q][jp][j] = sc * st[q][jp][j] + sum[q][jp][j];
+                        for (int u = 0; u < NU; ++u) {
+                            const f32x4 o = stl[((q * 2 + jp) * NU + u) * 64];
+                            const float v[4] = {sc * o.x + sum[q][jp][4 * u], sc * o.y + sum[q][jp][4 * u + 1],
+                                                sc * o.z + sum[q][jp][4 * u + 2], sc * o.w + sum[q][jp][4 * u + 3]};
+                            stl[((q * 2 + jp) * NU + u) * 64] = (f32x4){v[0], v[1], v[2], v[3]};
+                            store_row<4>(rs, dt_dst, vo, (2 * WV * q + jp) * pitch + 4 * u, v);
+                        }
+            } else {
+#pragma unroll
+                for (int q = 0; q < NOWN; ++q)
+#pragma unroll
+                    for (int jp = 0; jp < 2; ++jp)
+#pragma unroll
+                        for (int j = 0; j < NB; ++j) st[q][jp][j] = sc * st[q][jp][j] + sum[q][jp][j];
+            }
         }
         mcur = mnext;
     };
@@ -497,7 +547,7 @@ __global__ void __launch_bounds__(64 * WV, 2) mfma_kernel(const Params p)
             chunk(c, bZ, bX, bY); if (++c >= c_end) break;
         }
     }
-    if (FUSED) {
+    if (FUSED && !ST_LDS) {
 #pragma unroll
         for (int q = 0; q < NOWN; ++q)
 #pragma unroll
@@ -536,7 +586,7 @@ static hipError_t launch_one(const Params &p, dim3 grid, hipStream_t s)
 {
     const bool all32 = (!p.out || p.dt_out == DT_F32) && (!p.states || p.dt_states == DT_F32) &&
                        (!p.init || p.dt_init == DT_F32);
-    constexpr int lds = lds_bytes<NB, KS, WV>();
+    constexpr int lds = lds_bytes<NB, KS, WV, FUSED>();
     // more than 64 KB of LDS per workgroup has to be requested explicitly, once per kernel
     static bool configured[2] = {false, false};
     if (lds > 65536 && !configured[all32]) {
