@@ -117,6 +117,18 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
 int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
 
 /*
+ * dt preparation and per-chunk cumulative sum, the producer of `dt` and `dA_cumsum` for the three calls above.
+ * Replaces _chunk_cumsum_fwd / _chunk_cumsum_fwd_kernel (kernels/ssd_chunk_state.py:176-199, 33-79):
+ *   d = float(dt[b,l,h]) (+ dt_bias[h]); d = log1p(exp(d)) where dt_softplus and d <= 20; d = clamp(d, dt_min, dt_max);
+ *   d = 0 for tokens past seqlen;  dt_out[b,h,c,k] = d;  dA_cumsum[b,h,c,k] = sum_{j<=k} d_j * A[h].
+ * dt: (batch, seqlen, nheads) f32/bf16/f16, any strides; A, dt_bias (nullable): (nheads), f32/bf16/f16;
+ * dt_out, dA_cumsum: (batch, nheads, nchunks, chunk_size) fp32, any strides.  chunk_size <= 1024.
+ */
+int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *dt_out,
+                         const ssd_tensor *dA_cumsum, int32_t batch, int32_t seqlen, int32_t nheads, int32_t chunk_size,
+                         int dt_softplus, float dt_min, float dt_max, void *stream);
+
+/*
  * Tuning / test hook with no counterpart in the reference: how many waves split the tokens of a chunk in the bf16
  * MFMA kernels.  0 = let the library choose from the problem size (the default), 2 or 4 = force that split for
  * every later call of this process.  Returns the previous setting, or SSD_ERR_SHAPE for any other value.

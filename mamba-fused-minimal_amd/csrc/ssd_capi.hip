@@ -186,6 +186,36 @@ int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dim
     return ssd::mfma_supported(p) ? 1 : 0;
 }
 
+int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *dt_out,
+                         const ssd_tensor *dA_cumsum, int32_t batch, int32_t seqlen, int32_t nheads, int32_t chunk_size,
+                         int dt_softplus, float dt_min, float dt_max, void *stream)
+{
+    if (!present(dt) || !present(A) || !present(dt_out) || !present(dA_cumsum)) return SSD_ERR_NULL;
+    if (batch <= 0 || seqlen <= 0 || nheads <= 0 || chunk_size <= 0) return SSD_ERR_SHAPE;
+    if (!dtype_ok(dt->dtype) || !dtype_ok(A->dtype) || dt_out->dtype != SSD_F32 || dA_cumsum->dtype != SSD_F32)
+        return SSD_ERR_DTYPE;
+    ssd::CumsumParams p;
+    memset(&p, 0, sizeof(p));
+    p.dt = dt->data; p.dt_type = dt->dtype;
+    p.sdt_b = dt->stride[0]; p.sdt_l = dt->stride[1]; p.sdt_h = dt->stride[2];
+    p.A = A->data; p.A_type = A->dtype; p.sA = A->stride[0];
+    if (present(dt_bias)) {
+        if (!dtype_ok(dt_bias->dtype)) return SSD_ERR_DTYPE;
+        p.dt_bias = dt_bias->data; p.dt_bias_type = dt_bias->dtype; p.sbias = dt_bias->stride[0];
+    }
+    p.dt_out = (float *)dt_out->data;
+    p.so_b = dt_out->stride[0]; p.so_h = dt_out->stride[1]; p.so_c = dt_out->stride[2]; p.so_k = dt_out->stride[3];
+    p.dacs = (float *)dA_cumsum->data;
+    p.sa_b = dA_cumsum->stride[0]; p.sa_h = dA_cumsum->stride[1]; p.sa_c = dA_cumsum->stride[2]; p.sa_k = dA_cumsum->stride[3];
+    p.batch = batch; p.seqlen = seqlen; p.nheads = nheads; p.Q = chunk_size;
+    p.C = (seqlen + chunk_size - 1) / chunk_size;
+    p.softplus = dt_softplus ? 1 : 0; p.dt_min = dt_min; p.dt_max = dt_max;
+    if (!ssd::chunk_cumsum_supported(p)) return SSD_ERR_SHAPE;
+    int rc = check_device();
+    if (rc) return rc;
+    return (int)ssd::launch_chunk_cumsum(p, (hipStream_t)stream);
+}
+
 int ssd_set_token_split(int waves)
 {
     if (waves != 0 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;

@@ -52,6 +52,22 @@ struct PassParams {
     int dt_states, dt_out, dt_init;
 };
 
+// dt preparation + per-chunk cumulative sum.
+struct CumsumParams {
+    const void *dt;        // (b, L, H), any of the three element types
+    const void *A;         // (H)
+    const void *dt_bias;   // (H) or null
+    float *dt_out;         // (b, H, C, Q)
+    float *dacs;           // (b, H, C, Q)
+    int batch, seqlen, nheads, Q, C;
+    int64_t sdt_b, sdt_l, sdt_h, sA, sbias;
+    int64_t so_b, so_h, so_c, so_k;
+    int64_t sa_b, sa_h, sa_c, sa_k;
+    int dt_type, A_type, dt_bias_type;
+    int softplus;
+    float dt_min, dt_max;
+};
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t hbits) { return __builtin_bit_cast(float, hbits << 16); }
 
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
@@ -78,6 +94,8 @@ hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
+hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
+bool chunk_cumsum_supported(const CumsumParams &p);
 int set_token_split(int wv);      // 0 = automatic; 2 or 4 forces the token split of the MFMA kernels; returns the old value
 
 }  // namespace ssd

@@ -8,6 +8,7 @@ Same names, positional order, defaults, shape asserts and output shapes/dtypes a
 of the reference.  The wrappers own allocation and argument checking; the arithmetic runs in the gfx950 HIP
 kernels behind the C ABI of libssd_gfx950.so, asynchronously on the current torch stream."""
 import ctypes
+import math
 
 import torch
 
@@ -150,6 +151,28 @@ def _fused_chunk_state_state_passing_fwd_concurrent(B, x, dt, dA_cumsum, out_dty
     """Drop-in for kernels/fused_concurrent.py:255 (same signature and returns; prints nothing)."""
     return _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=initial_states,
                                                 seq_idx=seq_idx, states=states, states_in_fp32=states_in_fp32)
+
+
+def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """dt preparation + per-chunk cumulative sum of dt * A; same call surface as the reference's
+    kernels/ssd_chunk_state.py:176-199.  dt (batch, seqlen, nheads) -> (dA_cumsum, dt_out), both
+    (batch, nheads, nchunks, chunk_size) fp32."""
+    batch, seqlen, nheads = dt.shape
+    assert A.shape == (nheads,)
+    if dt_bias is not None:
+        assert dt_bias.shape == (nheads,)
+    _lib.require_device(dt, "_chunk_cumsum_fwd")
+    nchunks = math.ceil(seqlen / chunk_size)
+    dt_out = torch.empty(batch, nheads, nchunks, chunk_size, device=dt.device, dtype=torch.float32)
+    dA_cumsum = torch.empty(batch, nheads, nchunks, chunk_size, device=dt.device, dtype=torch.float32)
+    lib = _lib.load()
+    with torch.cuda.device(dt.device):
+        rc = lib.ssd_chunk_cumsum_fwd(_lib.tensor_arg(dt), _lib.tensor_arg(A), _lib.tensor_arg(dt_bias),
+                                      _lib.tensor_arg(dt_out), _lib.tensor_arg(dA_cumsum), batch, seqlen, nheads,
+                                      int(chunk_size), int(bool(dt_softplus)), float(dt_limit[0]), float(dt_limit[1]),
+                                      _stream(dt))
+    _lib.check(rc, "ssd_chunk_cumsum_fwd")
+    return dA_cumsum, dt_out
 
 
 def set_token_split(waves):

@@ -61,6 +61,16 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_query_path(_lib.tensor_arg(None), _lib.tensor_arg(B), dims) == -1
     odd = _lib.dims_arg(1, 256, 2, 40, 128, 1, 256, 1)                                     # headdim 40: generic
     assert lib.ssd_query_path(_lib.tensor_arg(x), _lib.tensor_arg(B), odd) == 0
+    # chunk cumsum: argument rejection happens before any device work
+    dt = torch.zeros(1, 256, 2)
+    A = torch.zeros(2)
+    o = torch.zeros(1, 2, 1, 256)
+    T = _lib.tensor_arg
+    assert lib.ssd_chunk_cumsum_fwd(T(None), T(A), T(None), T(o), T(o), 1, 256, 2, 256, 0, 0.0, 1.0, None) == -1
+    assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 256, 2, 0, 0, 0.0, 1.0, None) == -2
+    assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o.bfloat16()), T(o), 1, 256, 2, 256, 0, 0.0, 1.0, None) == -3
+    assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 4096, 2, 2048, 0, 0.0, 1.0, None) == -2   # chunk > 1024
+    assert lib.ssd_set_token_split(3) == -2 and lib.ssd_set_token_split(0) == 0
 
 
 def test_signatures_match_reference_call_surface():
@@ -76,6 +86,12 @@ def test_signatures_match_reference_call_surface():
     assert sig(ssd_amd._fused_chunk_state_state_passing_fwd_concurrent) == want
     d = inspect.signature(ssd_amd._chunk_state_fwd).parameters
     assert d["seq_idx"].default is None and d["states"].default is None and d["states_in_fp32"].default is True
+    # kernels/ssd_chunk_state.py:176
+    assert sig(ssd_amd._chunk_cumsum_fwd) == ["dt", "A", "chunk_size", "dt_bias", "dt_softplus", "dt_limit"]
+    d = inspect.signature(ssd_amd._chunk_cumsum_fwd).parameters
+    assert d["dt_bias"].default is None and d["dt_softplus"].default is False and d["dt_limit"].default == (0.0, float("inf"))
+    import kernels.ssd_chunk_state as k
+    assert k._chunk_cumsum_fwd is ssd_amd._chunk_cumsum_fwd and k._chunk_state_fwd is ssd_amd._chunk_state_fwd
 
 
 def test_shape_asserts_mirror_the_reference():
@@ -91,6 +107,10 @@ def test_shape_asserts_mirror_the_reference():
         ssd_amd._chunk_state_fwd(B, x, dt, dt, seq_idx=torch.zeros(1, 255, dtype=torch.int32))
     with pytest.raises(AssertionError):
         ssd_amd._chunk_state_fwd(B, x, dt, dt, states=torch.zeros(1, 1, 4, 64, 64))
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_cumsum_fwd(torch.zeros(1, 256, 4), torch.zeros(3), 256)              # A.shape != (nheads,)
+    with pytest.raises(AssertionError):
+        ssd_amd._chunk_cumsum_fwd(torch.zeros(1, 256, 4), torch.zeros(4), 256, dt_bias=torch.zeros(5))
     with pytest.raises(AssertionError):
         ssd_amd._state_passing_fwd(torch.zeros(1, 2, 4, 8), torch.zeros(1, 4, 3))
     with pytest.raises(AssertionError):

@@ -250,3 +250,49 @@ def test_reference_module_names_resolve(ops):
     from kernels.fused_concurrent import _fused_chunk_state_state_passing_fwd_concurrent
     assert _chunk_state_fwd is ops._chunk_state_fwd and _state_passing_fwd is ops._state_passing_fwd
     assert callable(_fused_chunk_state_state_passing_fwd_globalbar) and callable(_fused_chunk_state_state_passing_fwd_concurrent)
+
+
+# ------------------------------------------------------------------ dt preparation + per-chunk cumulative sum
+@pytest.mark.parametrize("kw", [
+    dict(),                                              # cfg 1 shape: bf16 dt, bias, softplus
+    dict(L=1000),                                        # ragged last chunk
+    dict(H=5, Q=64, L=512),                              # head count below one tile, chunk 64
+    dict(H=40, Q=128),                                   # two head tiles, the second partial
+    dict(Q=1024, L=4096, b=1),                           # the largest chunk the kernel takes (> 64 KB of LDS)
+    dict(dtype="fp32", b=1, L=1024),                     # fp32 dt
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
+def test_chunk_cumsum(ops, oracle, kw):
+    base = dict(b=2, L=2048, H=24)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    Q = d["cfg"]["Q"]
+    raw, A, bias = d["dt_raw"], d["A"], d["dt_bias"]
+    for softplus, use_bias, limit in ((True, True, (0.0, float("inf"))), (False, False, (0.0, float("inf"))),
+                                      (True, True, (2e-3, 5e-2))):
+        want_da, want_dt = oracle.chunk_cumsum_ref(raw, A, Q, dt_bias=bias if use_bias else None, dt_softplus=softplus,
+                                                   dt_limit=limit)
+        got_da, got_dt = ops._chunk_cumsum_fwd(_dev(raw), _dev(A), Q, dt_bias=_dev(bias) if use_bias else None,
+                                               dt_softplus=softplus, dt_limit=limit)
+        torch.cuda.synchronize()
+        assert got_dt.dtype == torch.float32 and got_da.dtype == torch.float32
+        _check(f"cumsum.dt[{softplus},{use_bias},{limit}]", got_dt, want_dt, 2e-6, 1e-9)
+        _check(f"cumsum.dA_cumsum[{softplus},{use_bias},{limit}]", got_da, want_da, 1e-5, 1e-6)
+
+
+def test_chunk_cumsum_strided_dt_and_pipeline(ops, oracle):
+    # dt as a strided slice of a packed projection, then the whole pipeline cumsum -> fused against the oracle
+    d = oracle.make_inputs(1, b=2, L=1024, H=6, init=True)
+    Q = d["cfg"]["Q"]
+    raw = d["dt_raw"]
+    packed = torch.zeros(raw.shape[0], raw.shape[1], raw.shape[2] + 10, dtype=raw.dtype)
+    packed[..., 7:7 + raw.shape[2]] = raw
+    view = _dev(packed)[..., 7:7 + raw.shape[2]]
+    assert not view.is_contiguous()
+    dA, dt = ops._chunk_cumsum_fwd(view, _dev(d["A"]), Q, dt_bias=_dev(d["dt_bias"]), dt_softplus=True)
+    _check("cumsum.strided.dt", dt, d["dt"], 2e-6, 1e-9)
+    _check("cumsum.strided.dA", dA, d["dA_cumsum"], 1e-5, 1e-6)
+    out, fin = ops._fused_chunk_state_state_passing_fwd(_dev(d["B"]), _dev(d["x"]), dt, dA, torch.float32,
+                                                        initial_states=_dev(d["initial_states"]))
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    _check("pipeline.out", out, want_out)
+    _check("pipeline.final", fin, want_fin)
