@@ -18,6 +18,10 @@ chunk_state_ref        kernels/ssd_chunk_state.py:97-173, 202-232
 state_passing_ref      kernels/ssd_state_passing.py:27-84, 87-115
 fused_ref              kernels/fused_globalbar.py:201-266, kernels/fused_concurrent.py:255-331
                        (same contract: chunk state followed by state passing)
+bmm_chunk_ref          kernels/ssd_bmm.py:31-134   (the step before the chunk scan; outside the path, used to
+chunk_scan_ref         kernels/ssd_chunk_scan.py:38-215   run the path inside a whole SSD forward, main.py:60-104)
+token_scan_ref         no counterpart in the reference: token-serial y_t = C_t . h_t + D x_t in fp64, which pins
+                       the chunked composition cumsum -> chunk state -> state passing -> bmm -> chunk scan.
 token_recurrence_ref   no counterpart in the reference: an independent, chunk-free
                        evaluation of the same linear recurrence used to pin the two
                        chunked functions.
@@ -224,6 +228,109 @@ def token_recurrence_ref(x, B, dt_tok, A, chunk_size, initial_states=None, seq_i
         if (t + 1) % chunk_size == 0 and (t + 1) // chunk_size < nchunks:
             out[:, (t + 1) // chunk_size] = h
     return out, h
+
+
+# --------------------------------------------------------------------------------------
+# The callers on either side of the path inside a whole SSD forward (main.py:60-104): restated so that the
+# library's kernels can be exercised in place, and pinned by a token-serial evaluation of y.
+# --------------------------------------------------------------------------------------
+def bmm_chunk_ref(a, b, chunk_size, seq_idx=None):
+    """Follows kernels/ssd_bmm.py:46-87 (non-causal, grouped form).  a, b (batch, L, G, K) ->
+    out (batch, C, G, Q, Q) fp32 with out[.., m, n] = sum_k a[cQ+m, g, k] * b[cQ+n, g, k]; rows / columns past the
+    end of the sequence are zero; entries whose tokens belong to different sequences are zero."""
+    batch, seqlen, ngroups, k = a.shape
+    assert b.shape == a.shape
+    nchunks = math.ceil(seqlen / chunk_size)
+    pad = nchunks * chunk_size - seqlen
+    af, bf = a.float(), b.float()
+    if pad:
+        af = F.pad(af, (0, 0, 0, 0, 0, pad))
+        bf = F.pad(bf, (0, 0, 0, 0, 0, pad))
+    af = af.reshape(batch, nchunks, chunk_size, ngroups, k)
+    bf = bf.reshape(batch, nchunks, chunk_size, ngroups, k)
+    out = torch.einsum("bcmgk,bcngk->bcgmn", af, bf)
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+        ids = seq_idx.long()
+        # padded rows get -1 and padded columns -2, so they never match (:79-80)
+        idm = F.pad(ids, (0, pad), value=-1).reshape(batch, nchunks, chunk_size)
+        idn = F.pad(ids, (0, pad), value=-2).reshape(batch, nchunks, chunk_size)
+        same = idm[:, :, :, None] == idn[:, :, None, :]
+        out = out * same[:, :, None].float()
+    return out
+
+
+def chunk_scan_ref(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=None):
+    """Follows kernels/ssd_chunk_scan.py:65-169 with IS_CAUSAL (the wrapper passes True, :213).
+    y[cQ+m] = scale_m * (C[cQ+m] . states[c]) + sum_{k<=m} cb[m,k] * exp(min(dAcs_m - dAcs_k, 0)) * dt_k * x[cQ+k] + D x,
+    scale_m = exp(dAcs_m) * [seq_idx[cQ+m] == seq_idx[cQ-1]] (the latter taken as 0 for the first chunk).
+    Returns (out, out_x) in fp32: with z, out_x is y and out is y * z * sigmoid(z); without, (y, None)."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, Q = dt.shape
+    _, _, ngroups, dstate = C.shape
+    assert nheads % ngroups == 0
+    assert cb.shape == (batch, nchunks, ngroups, Q, Q)
+    assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+    ratio = nheads // ngroups
+    pad = nchunks * Q - seqlen
+    xf, Cf = x.float(), C.float()
+    if pad:
+        xf = F.pad(xf, (0, 0, 0, 0, 0, pad))
+        Cf = F.pad(Cf, (0, 0, 0, 0, 0, pad))
+    xc = xf.reshape(batch, nchunks, Q, nheads, headdim)
+    Cc = Cf.reshape(batch, nchunks, Q, ngroups, dstate).repeat_interleave(ratio, dim=3)          # (b,c,Q,H,N)
+    dacs = dA_cumsum.float().permute(0, 2, 1, 3)                                                 # (b,c,H,Q)
+    dtc = dt.float().permute(0, 2, 1, 3)
+    # contribution of the state entering the chunk (:94-117)
+    scale = torch.exp(dacs)                                                                      # (b,c,H,Q)
+    if seq_idx is not None:
+        ids = F.pad(seq_idx.long(), (0, pad), value=-1).reshape(batch, nchunks, Q)
+        prev = torch.zeros(batch, nchunks, dtype=torch.long)
+        prev[:, 1:] = ids[:, :-1, -1]
+        scale = scale * (ids == prev[:, :, None])[:, :, None, :].float()
+    y = torch.einsum("bcmhn,bchpn->bcmhp", Cc, states.float()) * scale.permute(0, 1, 3, 2)[..., None]
+    # intra-chunk part (:119-148)
+    decay = torch.exp(torch.clamp(dacs[..., :, None] - dacs[..., None, :], max=0.0))            # (b,c,H,m,k)
+    causal = torch.tril(torch.ones(Q, Q, dtype=torch.bool))
+    cbh = cb.float().repeat_interleave(ratio, dim=2)                                             # (b,c,H,m,k)
+    m = cbh * decay * dtc[..., None, :] * causal.float()
+    y = y + torch.einsum("bchmk,bckhp->bcmhp", m, xc)
+    if D is not None:
+        Df = D.float()
+        y = y + xc * (Df[None, None, None, :, :] if Df.dim() == 2 else Df[None, None, None, :, None])
+    y = y.reshape(batch, nchunks * Q, nheads, headdim)[:, :seqlen]
+    if z is None:
+        return y, None
+    zf = z.float()
+    return y * zf * torch.sigmoid(zf), y
+
+
+def token_scan_ref(x, B, C, dt_tok, A, D=None, initial_states=None, seq_idx=None):
+    """Token-serial selective scan in fp64, with no notion of chunks:
+    h_t = [id_t == id_{t-1}] * exp(dt_t A_h) * h_{t-1} + dt_t * x_t (outer) B_t,  y_t = C_t . h_t + D x_t.
+    Returns (y (b, L, H, P), h_{L-1})."""
+    batch, seqlen, nheads, headdim = x.shape
+    ngroups, dstate = B.shape[2], B.shape[3]
+    ratio = nheads // ngroups
+    h = (torch.zeros(batch, nheads, headdim, dstate, dtype=torch.float64) if initial_states is None
+         else initial_states.double().clone())
+    xd, Bd, Cd, dtd, Ad = x.double(), B.double(), C.double(), dt_tok.double(), A.double()
+    y = torch.empty(batch, seqlen, nheads, headdim, dtype=torch.float64)
+    prev = torch.zeros(batch, dtype=torch.long)
+    for t in range(seqlen):
+        a = torch.exp(dtd[:, t] * Ad[None, :])
+        if seq_idx is not None:
+            cur = seq_idx[:, t].long()
+            a = a * (cur == prev)[:, None].double()
+            prev = cur
+        Bt = Bd[:, t].repeat_interleave(ratio, dim=1)
+        Ct = Cd[:, t].repeat_interleave(ratio, dim=1)
+        h = a[..., None, None] * h + dtd[:, t][..., None, None] * xd[:, t][..., None] * Bt[:, :, None, :]
+        y[:, t] = torch.einsum("bhpn,bhn->bhp", h, Ct)
+        if D is not None:
+            Dd = D.double()
+            y[:, t] += xd[:, t] * (Dd[None] if Dd.dim() == 2 else Dd[None, :, None])
+    return y, h
 
 
 # --------------------------------------------------------------------------------------

@@ -296,3 +296,27 @@ def test_chunk_cumsum_strided_dt_and_pipeline(ops, oracle):
     want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
     _check("pipeline.out", out, want_out)
     _check("pipeline.final", fin, want_fin)
+
+
+# ------------------------------------------------------------------ the path inside a whole SSD forward
+@pytest.mark.parametrize("kw", [dict(), dict(nseq=4, L=900, init=True)], ids=["plain", "varlen-ragged-init"])
+def test_whole_ssd_forward_with_library_kernels(ops, oracle, kw):
+    # main.py:78-103: cumsum -> fused chunk state + state passing run on the GPU through the library, the two
+    # stages after them (bmm, chunk scan) are the oracle's restatements; the result is compared with the
+    # token-serial selective scan, which knows nothing about chunks.
+    base = dict(b=1, L=1024, H=4, G=2)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    Q = d["cfg"]["Q"]
+    g = torch.Generator().manual_seed(11)
+    D = torch.randn(d["x"].shape[2], generator=g)
+    seq, init = d["seq_idx"], d["initial_states"]
+    dA, dt = ops._chunk_cumsum_fwd(_dev(d["dt_raw"]), _dev(d["A"]), Q, dt_bias=_dev(d["dt_bias"]), dt_softplus=True)
+    states, final = ops._fused_chunk_state_state_passing_fwd_globalbar(_dev(d["B"]), _dev(d["x"]), dt, dA, torch.float32,
+                                                                       initial_states=_dev(init), seq_idx=_dev(seq))
+    torch.cuda.synchronize()
+    cb = oracle.bmm_chunk_ref(d["C"], d["B"], Q, seq_idx=seq)
+    y, _ = oracle.chunk_scan_ref(cb, d["x"], dt.cpu(), dA.cpu(), d["C"], states.cpu(), D=D, seq_idx=seq)
+    y64, h64 = oracle.token_scan_ref(d["x"], d["B"], d["C"], d["dt_tok"], d["A"], D=D, initial_states=init, seq_idx=seq)
+    _check("forward.y", y, y64.float())
+    _check("forward.final", final, h64.float())

@@ -331,3 +331,80 @@ def test_make_inputs_shapes_and_distributions(oracle):
     assert torch.equal(d["x"], d2["x"]) and torch.equal(d["dt"], d2["dt"])
     c2 = oracle.CONFIGS[2]
     assert oracle.algorithmic_bytes(c2) == 721_420_288 and oracle.algorithmic_flops(c2) == 43_117_445_120
+
+
+# ---------------------------------------------------------------- the callers either side of the path
+def _ssd_forward_chunked(o, d, Cm, D, z, Q):
+    """main.py:78-103 with the oracle's restatements: cumsum -> fused -> bmm -> chunk scan."""
+    dA, dt = o.chunk_cumsum_ref(d["dt_raw"], d["A"], Q, dt_bias=d["dt_bias"], dt_softplus=True)
+    states, final = o.fused_ref(d["B"], d["x"], dt, dA, initial_states=d["initial_states"], seq_idx=d["seq_idx"])
+    cb = o.bmm_chunk_ref(Cm, d["B"], Q, seq_idx=d["seq_idx"])
+    out, out_x = o.chunk_scan_ref(cb, d["x"], dt, dA, Cm, states, D=D, z=z, seq_idx=d["seq_idx"])
+    return out, out_x, final
+
+
+@pytest.mark.parametrize("kw", [
+    dict(),
+    dict(nseq=3, L=200),                       # packed sequences + ragged last chunk
+    dict(G=2, init=True),                      # grouped B / C, initial states
+], ids=["base", "varlen-ragged", "groups-init"])
+def test_whole_forward_equals_token_serial_scan(oracle, kw):
+    o = oracle
+    base = dict(b=2, L=192, H=4, P=8, N=16, G=1, Q=64, dtype="fp32")
+    base.update(kw)
+    d = o.make_inputs(1, **base)
+    g = torch.Generator().manual_seed(7)
+    D = torch.randn(4, generator=g)
+    z = torch.randn(d["x"].shape, generator=g)
+    out, out_x, final = _ssd_forward_chunked(o, d, d["C"], D, z, 64)
+    y64, h64 = o.token_scan_ref(d["x"], d["B"], d["C"], d["dt_tok"], d["A"], D=D, initial_states=d["initial_states"],
+                                seq_idx=d["seq_idx"])
+    assert torch.allclose(out_x.double(), y64, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(out.double(), y64 * z.double() * torch.sigmoid(z.double()), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(final.double(), h64, rtol=1e-4, atol=1e-5)
+    # chunk-size invariance of the whole forward
+    out2, _, final2 = _ssd_forward_chunked(o, d, d["C"], D, z, 32)
+    assert torch.allclose(out2, out, rtol=1e-4, atol=1e-5) and torch.allclose(final2, final, rtol=1e-4, atol=1e-5)
+
+
+def test_bmm_chunk_brute_force_and_masks(oracle):
+    o = oracle
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(1, 10, 2, 3, generator=g)
+    b = torch.randn(1, 10, 2, 3, generator=g)
+    seq = torch.tensor([[0, 0, 0, 1, 1, 1, 1, 2, 2, 2]], dtype=torch.int32)
+    out = o.bmm_chunk_ref(a, b, 4, seq_idx=seq)          # 3 chunks, the last one ragged (2 tokens)
+    assert out.shape == (1, 3, 2, 4, 4)
+    for c in range(3):
+        for gi in range(2):
+            for m in range(4):
+                for n in range(4):
+                    tm, tn = 4 * c + m, 4 * c + n
+                    want = 0.0
+                    if tm < 10 and tn < 10 and seq[0, tm] == seq[0, tn]:
+                        want = float((a[0, tm, gi] * b[0, tn, gi]).sum())
+                    assert abs(float(out[0, c, gi, m, n]) - want) < 1e-5, (c, gi, m, n)
+
+
+def test_chunk_scan_special_cases(oracle):
+    o = oracle
+    b, L, H, P, N, Q = 1, 8, 2, 3, 4, 4
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(b, L, H, P, generator=g)
+    C = torch.randn(b, L, 1, N, generator=g)
+    states = torch.randn(b, 2, H, P, N, generator=g)
+    zeros = torch.zeros(b, H, 2, Q)
+    # dt = 0 and dA_cumsum = 0: no intra-chunk term, unit decay -> y[m] = C[m] . states[c]
+    cb = torch.randn(b, 2, 1, Q, Q, generator=g)
+    y, none = o.chunk_scan_ref(cb, x, zeros, zeros, C, states)
+    assert none is None
+    want = torch.einsum("bcmn,bchpn->bcmhp", C[:, :, 0].reshape(b, 2, Q, N), states).reshape(b, L, H, P)
+    assert torch.allclose(y, want, atol=1e-6)
+    # states = 0, dA_cumsum = 0, dt = 1: y[m] = sum_{k<=m} cb[m,k] x[k]  (causal), plus D x
+    ones = torch.ones(b, H, 2, Q)
+    D = torch.tensor([0.5, -2.0])
+    y, _ = o.chunk_scan_ref(cb, x, ones, zeros, C, torch.zeros_like(states), D=D)
+    for c in range(2):
+        for m in range(Q):
+            want = sum(cb[0, c, 0, m, k] * x[0, c * Q + k] for k in range(m + 1)) + x[0, c * Q + m] * D[:, None]
+            assert torch.allclose(y[0, c * Q + m], want, atol=1e-5)
