@@ -104,6 +104,23 @@ def main():
     wall_step, ev_step = timed(fused, args.steps, args.warmup)
     unf_wall, unf_ev = timed(unfused, max(5, args.steps // 4), 3)
 
+    # neighbours of the path, reported beside the headline: the fused call with bf16 passed states (what the
+    # reference's main.py asks for, out_dtype = C.dtype) and the producer of dt / dA_cumsum
+    def fused_bf16(i):
+        s = sets[i % nsets]
+        return ssd_amd._fused_chunk_state_state_passing_fwd(
+            s["B"], s["x"], s["dt"], s["dA_cumsum"], torch.bfloat16, initial_states=s["initial_states"],
+            seq_idx=s["seq_idx"])
+
+    raw = [mv(d["dt_raw"]).clone() for _ in range(nsets)]
+    A_dev, bias_dev = mv(d["A"]), mv(d["dt_bias"])
+
+    def cumsum(i):
+        return ssd_amd._chunk_cumsum_fwd(raw[i % nsets], A_dev, cfg["Q"], dt_bias=bias_dev, dt_softplus=True)
+
+    _, bf16_ev = timed(fused_bf16, max(5, args.steps // 4), 3)
+    _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
+
     # parity of what was timed, on one batch row, against the CPU oracle
     out, fin = fused(0)
     torch.cuda.synchronize()
@@ -142,6 +159,8 @@ def main():
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "unfused_us": round(unf_ev * 1e6, 2),
+        "fused_bf16_out_us": round(bf16_ev * 1e6, 2),
+        "chunk_cumsum_us": round(cs_ev * 1e6, 2),
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,
     }

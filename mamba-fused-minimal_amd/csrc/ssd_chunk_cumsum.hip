@@ -19,20 +19,13 @@ namespace {
 constexpr int kHeadTile = 32;
 constexpr int kMaxQ = 1024;
 
-__device__ __forceinline__ float wave_inclusive_scan(float v, int lane)
-{
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const float o = __shfl_up(v, d, 64);
-        if (lane >= d) v += o;
-    }
-    return v;
-}
-
+// EPL = tokens per lane in the scan = ceil(chunk_size / 64); VEC = outputs have unit stride along the chunk and
+// 16-byte aligned rows, so a lane's EPL = 4 results leave as one 16-byte store
+template <int EPL, bool VEC>
 __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
 {
-    extern __shared__ float tile[];                 // [kHeadTile][Q + 1]
-    const int Q = p.Q, pitch = Q + 1;
+    extern __shared__ __attribute__((aligned(16))) float tile[];     // [kHeadTile][Q + 4]: rows stay 16-byte aligned
+    const int Q = p.Q, pitch = Q + 4;
     const int b = blockIdx.z, c = blockIdx.y, h0 = blockIdx.x * kHeadTile;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lim = min(Q, p.seqlen - c * Q);
@@ -42,42 +35,91 @@ __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
     const int h = h0 + hh;
     const bool hv = h < p.nheads;
     const float bias = (hv && p.dt_bias) ? load_as_f32(p.dt_bias, (int64_t)h * p.sbias, p.dt_bias_type) : 0.f;
-    for (int k = tid / kHeadTile; k < Q; k += 256 / kHeadTile) {
+    // all of a thread's loads (up to 32 at a time) are issued before the first is used: the kernel is otherwise a
+    // chain of memory latencies
+    constexpr int NIT = 8 * EPL;                    // token rows per thread: chunk_size <= 64 * EPL
+    const char *dt_base = (const char *)p.dt;
+    const int64_t esz = p.dt_type == DT_F32 ? 4 : 2;
+    const int64_t off0 = (b * p.sdt_b + (int64_t)(c * Q + tid / kHeadTile) * p.sdt_l + (int64_t)h * p.sdt_h) * esz;
+    const int64_t step = 8 * p.sdt_l * esz;
+#pragma unroll 32
+    for (int i = 0; i < NIT; ++i) {
+        const int k = tid / kHeadTile + 8 * i;
+        if (k >= Q) break;
         float d = 0.f;
         if (hv && k < lim) {
-            d = load_as_f32(p.dt, b * p.sdt_b + (int64_t)(c * Q + k) * p.sdt_l + (int64_t)h * p.sdt_h, p.dt_type) + bias;
-            if (p.softplus && d <= 20.f) d = log1pf(expf(d));
+            d = load_as_f32(dt_base + off0 + i * step, 0, p.dt_type) + bias;
+            if (p.softplus && d <= 20.f) {
+                // log1p(t) = log(u) * t / (u - 1) with u = fl(1 + t): the quotient compensates the rounding of u,
+                // so the hardware exp / log instructions suffice (a libm log1pf made this kernel ALU-bound)
+                const float t = __expf(d), u = 1.f + t;
+                d = u == 1.f ? t : __logf(u) * __fdividef(t, u - 1.f);
+            }
             d = fminf(fmaxf(d, p.dt_min), p.dt_max);
         }
         tile[hh * pitch + k] = d;
     }
     __syncthreads();
 
-    // ---- per head row: scan and store
-    const int epl = (Q + 63) >> 6;                  // tokens per lane
-    for (int r = wave; r < kHeadTile; r += 4) {
-        const int hr = h0 + r;
-        if (hr >= p.nheads) break;                  // wave-uniform
-        const float a = load_as_f32(p.A, (int64_t)hr * p.sA, p.A_type);
-        const float *row = tile + r * pitch;
-        float v[kMaxQ / 64];
-        float run = 0.f;
+    // ---- per head row: scan and store.  A wave owns rows wave, wave + 4, ...; NR of them are processed together
+    // so that the cross-lane steps of their scans overlap instead of queueing behind one another.
+    constexpr int NR = EPL <= 4 ? 8 : 2;
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    for (int r0 = wave; r0 < kHeadTile; r0 += 4 * NR) {
+        float dv[NR][EPL], v[NR][EPL], run[NR], tot[NR];
 #pragma unroll
-        for (int e = 0; e < kMaxQ / 64; ++e) {
-            const int k = lane * epl + e;
-            const float d = (e < epl && k < Q) ? row[k] : 0.f;
-            run += d * a;
-            v[e] = run;
+        for (int i = 0; i < NR; ++i) {
+            const int r = r0 + 4 * i, hr = h0 + r;
+            const bool valid = r < kHeadTile && hr < p.nheads;           // wave-uniform
+            const float a = valid ? load_as_f32(p.A, (int64_t)hr * p.sA, p.A_type) : 0.f;
+            const float *row = tile + (valid ? r : 0) * pitch;
+            if constexpr (VEC && EPL == 4) {
+                const f32x4 q = 4 * lane < Q ? *(const f32x4 *)(row + 4 * lane) : (f32x4){0.f, 0.f, 0.f, 0.f};
+                dv[i][0] = q.x; dv[i][1] = q.y; dv[i][2] = q.z; dv[i][3] = q.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    const int k = lane * EPL + e;
+                    dv[i][e] = k < Q ? row[k] : 0.f;
+                }
+            }
+            run[i] = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                run[i] += dv[i][e] * a;
+                v[i][e] = run[i];
+            }
+            tot[i] = run[i];
         }
-        const float before = wave_inclusive_scan(run, lane) - run;     // total of the lanes to the left
-        float *dt_out = p.dt_out + b * p.so_b + (int64_t)hr * p.so_h + (int64_t)c * p.so_c;
-        float *da_out = p.dacs + b * p.sa_b + (int64_t)hr * p.sa_h + (int64_t)c * p.sa_c;
 #pragma unroll
-        for (int e = 0; e < kMaxQ / 64; ++e) {
-            const int k = lane * epl + e;
-            if (e < epl && k < Q) {
-                dt_out[(int64_t)k * p.so_k] = row[k];
-                da_out[(int64_t)k * p.sa_k] = v[e] + before;
+        for (int d = 1; d < 64; d <<= 1)
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const float o = __shfl_up(tot[i], d, 64);
+                if (lane >= d) tot[i] += o;
+            }
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int r = r0 + 4 * i, hr = h0 + r;
+            if (r >= kHeadTile || hr >= p.nheads) continue;               // wave-uniform
+            const float before = tot[i] - run[i];                         // total of the lanes to the left
+            float *dt_out = p.dt_out + b * p.so_b + (int64_t)hr * p.so_h + (int64_t)c * p.so_c;
+            float *da_out = p.dacs + b * p.sa_b + (int64_t)hr * p.sa_h + (int64_t)c * p.sa_c;
+            if constexpr (VEC && EPL == 4) {
+                if (4 * lane < Q) {         // chunk_size is a multiple of 4 here
+                    *(f32x4 *)(dt_out + 4 * lane) = (f32x4){dv[i][0], dv[i][1], dv[i][2], dv[i][3]};
+                    *(f32x4 *)(da_out + 4 * lane) =
+                        (f32x4){v[i][0] + before, v[i][1] + before, v[i][2] + before, v[i][3] + before};
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    const int k = lane * EPL + e;
+                    if (k < Q) {
+                        dt_out[(int64_t)k * p.so_k] = dv[i][e];
+                        da_out[(int64_t)k * p.sa_k] = v[i][e] + before;
+                    }
+                }
             }
         }
     }
@@ -85,19 +127,33 @@ __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
 
 }  // namespace
 
-hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s)
+template <int EPL, bool VEC>
+static hipError_t launch_t(const CumsumParams &p, dim3 grid, size_t lds, hipStream_t s)
 {
-    dim3 grid((p.nheads + kHeadTile - 1) / kHeadTile, p.C, p.batch);
-    const size_t lds = (size_t)kHeadTile * (p.Q + 1) * sizeof(float);
-    static bool big_lds = false;        // more than 64 KB of LDS has to be requested explicitly, once
+    static bool big_lds = false;        // more than 64 KB of LDS has to be requested explicitly, once per kernel
     if (lds > 65536 && !big_lds) {
-        hipError_t e = hipFuncSetAttribute((const void *)chunk_cumsum_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           kHeadTile * (kMaxQ + 1) * (int)sizeof(float));
+        hipError_t e = hipFuncSetAttribute((const void *)chunk_cumsum_kernel<EPL, VEC>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kHeadTile * (kMaxQ + 4) * (int)sizeof(float));
         if (e != hipSuccess) return e;
         big_lds = true;
     }
-    hipLaunchKernelGGL(chunk_cumsum_kernel, grid, dim3(256), lds, s, p);
+    hipLaunchKernelGGL((chunk_cumsum_kernel<EPL, VEC>), grid, dim3(256), lds, s, p);
     return hipGetLastError();
+}
+
+hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s)
+{
+    dim3 grid((p.nheads + kHeadTile - 1) / kHeadTile, p.C, p.batch);
+    const size_t lds = (size_t)kHeadTile * (p.Q + 4) * sizeof(float);
+    const int epl = (p.Q + 63) / 64;
+    const bool vec = p.Q % 4 == 0 && p.so_k == 1 && p.sa_k == 1 && ((uintptr_t)p.dt_out | (uintptr_t)p.dacs) % 16 == 0 &&
+                     (p.so_b | p.so_h | p.so_c | p.sa_b | p.sa_h | p.sa_c) % 4 == 0;
+    if (epl == 1) return launch_t<1, false>(p, grid, lds, s);
+    if (epl == 2) return launch_t<2, false>(p, grid, lds, s);
+    if (epl <= 4) return vec && epl == 4 ? launch_t<4, true>(p, grid, lds, s) : launch_t<4, false>(p, grid, lds, s);
+    if (epl <= 8) return launch_t<8, false>(p, grid, lds, s);
+    return launch_t<16, false>(p, grid, lds, s);
 }
 
 bool chunk_cumsum_supported(const CumsumParams &p) { return p.Q >= 1 && p.Q <= kMaxQ && p.C <= 65535 && p.batch <= 65535; }
