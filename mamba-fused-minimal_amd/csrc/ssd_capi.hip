@@ -10,6 +10,8 @@ namespace {
 using ssd::Params;
 using ssd::PassParams;
 
+int g_forced_split = 0;     // ssd_set_token_split: a forced split also forces the token-split kernels
+
 bool dtype_ok(int dt) { return dt == SSD_F32 || dt == SSD_BF16 || dt == SSD_F16; }
 
 // Device check, cached per device ordinal: the kernels are gfx950 code objects only.
@@ -77,7 +79,13 @@ int run(const Params &p, bool fused, void *stream)
     int rc = check_device();
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    hipError_t e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
+    hipError_t e;
+    // Fused launch: with at least two state tiles per compute unit the four-tiles-per-workgroup kernel wins (B is
+    // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
+    // kernel, which puts four waves on every tile, has the shorter chunk.
+    const int tiles = p.batch * p.nheads * (p.headdim / 32);
+    if (fused && g_forced_split == 0 && tiles >= 512 && ssd::quad_supported(p)) e = ssd::launch_quad(p, s);
+    else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
     return (int)e;
 }
 
@@ -219,6 +227,7 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
 int ssd_set_token_split(int waves)
 {
     if (waves != 0 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;
+    g_forced_split = waves;
     return ssd::set_token_split(waves);
 }
 

@@ -94,6 +94,8 @@ hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
+hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state tiles per workgroup sharing B in LDS
+bool quad_supported(const Params &p);
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 int set_token_split(int wv);      // 0 = automatic; 2 or 4 forces the token split of the MFMA kernels; returns the old value

@@ -1,0 +1,474 @@
+// Fused chunk-state + state-passing kernel: four state tiles per workgroup, B shared through LDS (gfx950).
+//
+// A workgroup is four waves; each wave owns the (32 headdim rows) x (all dstate columns) tile of one
+// (batch, head, row slice) and walks the whole sequence, the four tiles sharing one (batch, group) and therefore
+// the same B rows.  The running state lives in the MFMA accumulators: at a chunk boundary a wave stores them as
+// out[:, c] (the state entering chunk c), multiplies them by exp(dA_chunk) -- or by zero where seq_idx changes --
+// and the chunk's 32-token steps accumulate sum_k B_k (x*w)_k on top: s <- exp(dA_chunk) * s + states_c
+// (kernels/ssd_state_passing.py:69-84 applied to the contraction of kernels/ssd_chunk_state.py:134-173).  There is
+// no token split, no LDS reduction and the per-chunk `states` tensor never exists, so callers that ask for it get
+// the token-split kernel instead.
+//
+// Data movement per 32-token step:
+//   * B: the step's 32 x dstate tile is fetched ONCE per workgroup, straight into a ring in LDS (buffer loads with
+//     LDS destination, each wave a quarter of the tile), three steps ahead.  The MFMA computes the state
+//     transposed, D[n][p] = sum_k B[k][n] * xw[k][p], so B is the A operand: lane (i, kg) needs the 8 tokens
+//     8kg..8kg+7 of column 16*it + i.  ds_read_b64_tr_b16 delivers exactly that from the row-major tile: within a
+//     16-lane group, lane i receives 16-bit element i%4 of the 8-byte words addressed by lanes i/4, i/4+4, i/4+8,
+//     i/4+12; with lane s addressing (token 4*half + s/4, columns 4*(s%4)..+3) lane i ends up with four consecutive
+//     tokens of column i.  No v_perm, no B registers, a quarter of the vector-memory instructions.
+//   * x: each wave fetches its own rows into a private four-slot LDS ring, three steps ahead, reads them back as
+//     (token, row pair) dwords, scales by the per-token weight in fp32 and splits into bf16 hi + bf16 lo (two MFMAs
+//     keep ~16 mantissa bits of x*w); the operands of step g+1 are prepared while the MFMAs of step g run.
+//   * out: accumulator register r of tile (it, jp) is dstate column 16*it + 4*kg + r of headdim row 2*j + jp, so
+//     the four registers of a tile are one 16-byte store and the state never moves between registers.
+// One s_barrier per step orders the shared ring: a wave passes it after its own part of the step's B tile has
+// landed and after it has finished reading the previous step's tile.
+#include "ssd_params.h"
+
+#include <utility>
+
+namespace ssd {
+
+namespace quad {
+
+// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ int esize_of(int dt) { return dt == DT_F32 ? 4 : 2; }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0x7fffffffLL ? 0x7fffffffLL : bytes),
+                                             0x00020000);
+}
+
+// s_waitcnt immediate that only waits for the vector-memory counter to drop to n (gfx9 field layout)
+constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
+// Four consecutive state values of one row -> fp32 / bf16 / f16 destination.  The data registers of a wide store
+// are read out over several cycles after issue; wait states that depend on them keep a following writer of the
+// same registers (here the decay multiplication of the accumulators) away.
+__device__ __forceinline__ void store4(__amdgpu_buffer_rsrc_t rs, int dt, int voff, int soff, f32x4 v)
+{
+    if (dt == DT_F32) {
+        const u32x4 q = __builtin_bit_cast(u32x4, v);
+        __builtin_amdgcn_raw_buffer_store_b128(q, rs, 4 * voff, 4 * soff, 0);
+        asm volatile("s_nop 3" ::"v"(q) : "memory");
+    } else if (dt == DT_BF16) {
+        const u32x2 q = {pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+        __builtin_amdgcn_raw_buffer_store_b64(q, rs, 2 * voff, 2 * soff, 0);
+        asm volatile("s_nop 3" ::"v"(q) : "memory");
+    } else {
+        typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+        const h2 a = {(_Float16)v.x, (_Float16)v.y}, c = {(_Float16)v.z, (_Float16)v.w};
+        const u32x2 q = {__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, c)};
+        __builtin_amdgcn_raw_buffer_store_b64(q, rs, 2 * voff, 2 * soff, 0);
+        asm volatile("s_nop 3" ::"v"(q) : "memory");
+    }
+}
+
+struct Frag { uint32_t hi[2][4], lo[2][4]; };
+
+constexpr int kRing = 4;            // steps of B kept in LDS (requested three steps ahead)
+
+template <int NT, int SPC> constexpr int wave_lds() { return 4 * 2048 + 3 * 32 * SPC * 4; }     // x ring + weights
+template <int NT, int SPC> constexpr int lds_bytes() { return kRing * NT * 1024 + 4 * wave_lds<NT, SPC>(); }
+
+// NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (chunk_size / 32: 4 or 8);
+// F32IO = out and initial states are fp32 (or the latter absent): element-type branches fold away.
+template <int NT, int SPC, bool HAS_SEQ, bool F32IO>
+__global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
+{
+    constexpr int Q = 32 * SPC;
+    constexpr int TPL = Q / 64;         // tokens per lane when the chunk's weights are computed (2 or 4)
+    constexpr int NTW = NT / 4;         // B tile blocks (32 tokens x 16 columns, 1 KB) a wave fetches per step
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    char *bring = lds;                                                   // kRing x NT blocks of 1 KB, shared
+    char *xring = lds + kRing * NT * 1024 + wave * wave_lds<NT, SPC>();  // 4 slots x (32 tokens x 64 bytes)
+    char *wbuf = xring + 4 * 2048;                                       // 3 slots x Q weights
+
+    // Work item -> (batch, head, row slice); the four items of a workgroup share batch and group (checked on the
+    // host).  Consecutive workgroups sit on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so a
+    // batch's B is fetched from HBM by one or two L2 slices only.
+    const int per_xcd = ((p.n_items >> 2) + 7) >> 3;                     // workgroups per XCD
+    const int wg = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (4 * wg >= p.n_items) return;                                     // whole workgroup: no barrier is skipped
+    const int item = 4 * wg + wave;
+    const int n_pt = p.headdim >> 5;
+    const int pt = item % n_pt;
+    const int r1 = item / n_pt;
+    const int h = r1 % p.nheads;
+    const int b = r1 / p.nheads;
+    const int C = p.C, L = p.seqlen;
+    const int g = h / (p.nheads / p.ngroups);
+    const int p0 = pt * 32;
+    const int dt_out = F32IO ? (int)DT_F32 : p.dt_out, dt_init = F32IO ? (int)DT_F32 : p.dt_init;
+
+    const char *xrow = (const char *)p.x + 2 * (b * p.sx_b + h * p.sx_h);
+    const char *Brow = (const char *)p.B + 2 * (b * p.sB_b + g * p.sB_g);
+    const int64_t xrb = 2 * p.sx_l, Brb = 2 * p.sB_l;            // row pitch in bytes
+    // descriptor of chunk c: base = its first token, extent = the tokens that exist (none past the last chunk)
+    auto chunk_rsrc = [&](const char *base, int64_t pitch, int c) {
+        const int cc = c < C ? c : 0;
+        return make_rsrc(base + (int64_t)cc * Q * pitch, c < C ? (int64_t)(L - c * Q) * pitch : 0);
+    };
+    const float *dtb = p.dt + b * p.sdt_b + h * p.sdt_h;
+    const float *dab = p.dacs + b * p.sda_b + h * p.sda_h;
+    const int32_t *sqb = HAS_SEQ ? p.seq + b * p.ssq_b : nullptr;
+
+    // ---- request helpers -------------------------------------------------------------------------------------
+    // B block `it` of a step = 32 tokens x 16 columns (32 bytes per token), 64 pieces of 16 bytes; lane l deposits
+    // its piece at byte 16*l of the block.  Piece l = (column half l/32, token bit 2 = (l/16)%2, position l%16) with
+    // token = position%4 + 4*((l/16)%2) + 8*(position/4): the 16 tokens that one transposing read touches then
+    // lie at the 16 different positions, i.e. on different LDS banks.
+    const int Blane = (int)(((lane & 3) | (((lane >> 4) & 1) << 2) | (((lane >> 2) & 3) << 3)) * Brb) + 16 * (lane >> 5);
+    auto load_B = [&](__amdgpu_buffer_rsrc_t rs, int s, int it) {       // step s of the chunk behind rs
+#if defined(__HIP_DEVICE_COMPILE__)      // the LDS address space does not exist in the host pass
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRing) * NT + it) * 1024), 16, Blane,
+                                                 (int)(32 * s * Brb) + 32 * it, 0, 0);
+#else
+        (void)rs; (void)s; (void)it; (void)Blane;
+#endif
+    };
+    // The transposing read for (block it, tokens 8kg + 4*half .. +3): lane (i16, kg) addresses the 8 bytes of
+    // token 8kg + 4*half + i16/4, columns 4*(i16%4)..+3 and receives column i16 of those four tokens.
+    // The reads are written as inline assembly with explicit s_waitcnt: given the intrinsic, the compiler orders
+    // every such read behind ALL outstanding loads that write LDS (s_waitcnt vmcnt(0)), which would serialise the
+    // three-steps-ahead requests with their use.
+    uint32_t Btr = (((i16 & 3) >> 1) * 2) * 256 + ((i16 >> 2) | (kg << 2)) * 16 + (i16 & 1) * 8;   // + 256 * half
+#if defined(__HIP_DEVICE_COMPILE__)
+    Btr += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
+#endif
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wunused-lambda-capture"   // the host pass sees no use of Btr
+    auto read_Bt = [&, Btr](auto offc, u32x2 &lo, u32x2 &hi) {        // offc: byte offset of the block in the ring
+        constexpr int off = decltype(offc)::value;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                     : "=&v"(lo), "=&v"(hi) : "v"(Btr), "n"(off), "n"(off + 256) : "memory");
+#else
+        lo = hi = (u32x2){0u, 0u}; (void)Btr; (void)off;
+#endif
+    };
+#pragma clang diagnostic pop
+    // results of read_Bt become valid here (and every other LDS operation of the wave is complete)
+    auto wait_Bt = [&](u32x2 &lo, u32x2 &hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi) : : "memory");
+#else
+        (void)lo; (void)hi;
+#endif
+    };
+    // x: two requests cover the 32 token rows of a step, 4 lanes per 64-byte row of the slice; lane l deposits
+    // its 16 bytes at byte 16*l of a 1 KB block.  Request i fetches tokens 8*kg' + 4*i + m into row slot
+    // 4*m + kg' (kg' = (l/4)%4, m = l/16), so the four kg groups of an operand read below hit different banks.
+    const int xlane = (int)((8 * ((lane >> 2) & 3) + (lane >> 4)) * xrb) + 2 * p0 + 16 * (lane & 3);
+    auto load_x = [&](__amdgpu_buffer_rsrc_t rs, int s, int i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xring + (s & 3) * 2048 + i * 1024), 16, xlane,
+                                                 (int)((32 * s + 4 * i) * xrb), 0, 0);
+#else
+        (void)rs; (void)s; (void)i; (void)xlane;
+#endif
+    };
+    const int xst_rd = 64 * kg + 4 * i16;     // + 2048 * slot + 1024 * (j/4) + 256 * (j%4) for token 8kg + j
+
+    // decay inputs of a chunk: TPL consecutive tokens per lane, plus the chunk-level scalars
+    struct Meta { float dtv[TPL], cs[TPL], last; int32_t id[TPL], id_last; };
+    auto load_meta = [&](int c) {
+        Meta m;
+        const int cc = c < C ? c : C - 1;
+        const float *dtp = dtb + cc * p.sdt_c + TPL * lane;
+        const float *dap = dab + cc * p.sda_c + TPL * lane;
+        if constexpr (TPL == 4) {
+            const f32x4 a = *(const f32x4 *)dtp, d = *(const f32x4 *)dap;
+            m.dtv[0] = a.x; m.dtv[1] = a.y; m.dtv[2] = a.z; m.dtv[3] = a.w;
+            m.cs[0] = d.x; m.cs[1] = d.y; m.cs[2] = d.z; m.cs[3] = d.w;
+        } else {
+            const f32x2 a = *(const f32x2 *)dtp, d = *(const f32x2 *)dap;
+            m.dtv[0] = a.x; m.dtv[1] = a.y; m.cs[0] = d.x; m.cs[1] = d.y;
+        }
+        m.last = dab[cc * p.sda_c + (Q - 1)];
+        m.id_last = 0;
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) m.id[t] = 0;
+        if (HAS_SEQ) {
+#pragma unroll
+            for (int t = 0; t < TPL; ++t) m.id[t] = sqb[(int64_t)min(cc * Q + TPL * lane + t, L - 1) * p.ssq_l];
+            m.id_last = sqb[(int64_t)(min((cc + 1) * Q, L) - 1) * p.ssq_l];
+        }
+        return m;
+    };
+    // per-token weights of chunk c (kernels/ssd_chunk_state.py:134-156) -> weight slot ws
+    auto put_weights = [&](int c, int ws, const Meta &m) {
+        float w[TPL];
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) {
+            float e = m.last - m.cs[t];
+            if (p.clamp) e = fminf(e, 0.f);
+            w[t] = __expf(e) * m.dtv[t];
+            if (c * Q + TPL * lane + t >= L) w[t] = 0.f;
+            if (HAS_SEQ && m.id[t] != m.id_last) w[t] = 0.f;
+        }
+        if constexpr (TPL == 4) *(f32x4 *)(wbuf + ws * Q * 4 + 16 * lane) = (f32x4){w[0], w[1], w[2], w[3]};
+        else *(f32x2 *)(wbuf + ws * Q * 4 + 8 * lane) = (f32x2){w[0], w[1]};
+    };
+
+    // ---- operand helpers -------------------------------------------------------------------------------------
+    // x dwords (token, headdim row pair i16) and weights of the 8 tokens 8kg..8kg+7 of step s
+    auto read_operands = [&](int s, int ws, uint32_t (&xr)[8], float (&wv)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            xr[j] = *(const uint32_t *)(xring + (s & 3) * 2048 + xst_rd + 1024 * (j >> 2) + 256 * (j & 3));
+        const f32x4 wlo = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg));
+        const f32x4 whi = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg + 4));
+        wv[0] = wlo.x; wv[1] = wlo.y; wv[2] = wlo.z; wv[3] = wlo.w;
+        wv[4] = whi.x; wv[5] = whi.y; wv[6] = whi.z; wv[7] = whi.w;
+    };
+    // tokens (2q, 2q+1) of headdim row 2*i16 + jp: x * w in fp32, split into bf16 hi + bf16 lo
+    auto frag_piece = [&](int q, int jp, const uint32_t (&xr)[8], const float (&wv)[8], Frag &f) {
+        const uint32_t r0 = xr[2 * q], r1_ = xr[2 * q + 1];
+        const float v0 = __builtin_bit_cast(float, jp ? (r0 & 0xffff0000u) : (r0 << 16)) * wv[2 * q];
+        const float v1 = __builtin_bit_cast(float, jp ? (r1_ & 0xffff0000u) : (r1_ << 16)) * wv[2 * q + 1];
+        const uint32_t hp = pack_bf16(v0, v1);
+        const float h0 = __builtin_bit_cast(float, hp << 16);
+        const float h1 = __builtin_bit_cast(float, hp & 0xffff0000u);
+        f.hi[jp][q] = hp;
+        f.lo[jp][q] = pack_bf16(v0 - h0, v1 - h1);
+    };
+
+    // ---- state ---------------------------------------------------------------------------------------------
+    // acc[it][jp][r]: dstate column 16*it + 4*kg + r of headdim row p0 + 2*i16 + jp
+    f32x4 acc[NT][2];
+    const int64_t slice_out = (int64_t)(p.headdim - 1) * p.so_p + p.dstate;
+    const int64_t slice_fin = (int64_t)(p.headdim - 1) * p.sf_p + p.dstate;
+    auto store_state = [&](__amdgpu_buffer_rsrc_t rs, int dt, int row_pitch) {
+        const int voff = (p0 + 2 * i16) * row_pitch + 4 * kg;
+#pragma unroll
+        for (int it = 0; it < NT; ++it)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp) store4(rs, dt, voff, jp * row_pitch + 16 * it, acc[it][jp]);
+    };
+#pragma unroll
+    for (int it = 0; it < NT; ++it)
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp) {
+            acc[it][jp] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            if (p.init) {
+                const int64_t off = b * p.sin_b + h * p.sin_h + (int64_t)(p0 + 2 * i16 + jp) * p.sin_p + 16 * it + 4 * kg;
+                if (dt_init == DT_F32) {
+                    acc[it][jp] = *(const f32x4 *)((const float *)p.init + off);
+                } else {
+                    const uint16_t *src = (const uint16_t *)p.init + off;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc[it][jp][r] = dt_init == DT_BF16 ? bf16_bits_to_f32(src[r])
+                                                            : (float)__builtin_bit_cast(_Float16, src[r]);
+                }
+            }
+        }
+
+    // ---- prologue: rows past the end of the sequence are not fetched and leave their LDS slots untouched; their
+    // weight is zero, so the slots only have to hold finite numbers.
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *(u32x4 *)(xring + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < kRing * NTW; ++i)
+        *(u32x4 *)(bring + (i * 4 + wave) * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): the zeros are in place before any row lands
+    __builtin_amdgcn_s_barrier();
+    Meta mcur = load_meta(0);
+    __amdgpu_buffer_rsrc_t rsx0 = chunk_rsrc(xrow, xrb, 0), rsx1 = chunk_rsrc(xrow, xrb, 1);
+    __amdgpu_buffer_rsrc_t rsB0 = chunk_rsrc(Brow, Brb, 0), rsB1 = chunk_rsrc(Brow, Brb, 1);
+    // requests of the steps 0..2, in the order (x, x, B...) that every later step keeps
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        load_x(rsx0, s, 0); load_x(rsx0, s, 1);
+#pragma unroll
+        for (int k = 0; k < NTW; ++k) load_B(rsB0, s, wave * NTW + k);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    put_weights(0, 0, mcur);
+    Frag fA, fB;
+    {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * (2 + NTW) - 2));      // the two x requests of step 0
+        asm volatile("" ::: "memory");
+        uint32_t xr[8]; float wv[8];
+        read_operands(0, 0, xr, wv);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { frag_piece(q, 0, xr, wv, fA); frag_piece(q, 1, xr, wv, fA); }
+    }
+    int32_t prev_id = 0;
+    Meta mnext = mcur;
+
+    // One 32-token step s of chunk c (weight slot ws): fc = x operands of this step, fn receives those of step + 1.
+    auto step = [&](int c, auto sc, int ws, Frag &fc, Frag &fn) {
+        constexpr int s = decltype(sc)::value;
+        // This step needs its B tile (every wave's part of it) and, for the next step's operands, this wave's x
+        // rows of step + 1.  A step issues its vector-memory requests in the order x, x, B.. (three steps ahead);
+        // memory operations complete in order, so this wave's B part (requested three steps ago) and the x rows of
+        // step + 1 (two steps ago) have landed once no more than the NTW B requests of that step and the 2 + NTW
+        // requests of the step in between are outstanding.  The compiler does not track loads that write LDS, so
+        // the wait is explicit; the barrier then publishes every wave's part and tells that all waves are done
+        // reading the tile of the previous step, whose ring slot this step's requests overwrite.
+        constexpr int kAfter = NTW + (2 + NTW);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kAfter));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        uint32_t xr[8]; float wv[8];
+        if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
+        else read_operands(0, (ws + 1) % 3, xr, wv);
+
+        if (s == 0) {
+            // chunk boundary: out[:, c] = state entering the chunk, then s <- exp(dA_chunk) * s
+            store_state(make_rsrc((char *)p.out + (b * p.so_b + c * p.so_c + h * p.so_h) * esize_of(dt_out),
+                                  slice_out * esize_of(dt_out)), dt_out, (int)p.so_p);
+            float sc = __expf(mcur.last);
+            if (HAS_SEQ) {
+                if (mcur.id_last != prev_id) sc = 0.f;
+                prev_id = mcur.id_last;
+            }
+#pragma unroll
+            for (int it = 0; it < NT; ++it)
+#pragma unroll
+                for (int jp = 0; jp < 2; ++jp) acc[it][jp] *= sc;
+        }
+        // requests of this step: x rows and this wave's B blocks of step + 3 (this chunk or the next)
+        const auto rsB = s + 3 < SPC ? rsB0 : rsB1;
+        const auto rsx = s + 3 < SPC ? rsx0 : rsx1;
+        const int s3 = (s + 3) % SPC;
+        const bf16x8 h0 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[0][0], fc.hi[0][1], fc.hi[0][2], fc.hi[0][3]});
+        const bf16x8 h1 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[1][0], fc.hi[1][1], fc.hi[1][2], fc.hi[1][3]});
+        const bf16x8 l0 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[0][0], fc.lo[0][1], fc.lo[0][2], fc.lo[0][3]});
+        const bf16x8 l1 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[1][0], fc.lo[1][1], fc.lo[1][2], fc.lo[1][3]});
+        u32x2 blo[2], bhi[2];            // B operand of tile it in slot it % 2, the next one in flight in the other
+        read_Bt(std::integral_constant<int, ((s % kRing) * NT) * 1024>{}, blo[0], bhi[0]);
+        __builtin_amdgcn_sched_barrier(0);   // operand reads above, the requests that reuse their slots below
+        static_for<NT>([&](auto itc) {
+            constexpr int it = decltype(itc)::value;
+            wait_Bt(blo[it & 1], bhi[it & 1]);
+            const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it & 1].x, blo[it & 1].y, bhi[it & 1].x, bhi[it & 1].y});
+            if constexpr (it + 1 < NT)
+                read_Bt(std::integral_constant<int, ((s % kRing) * NT + it + 1) * 1024>{}, blo[(it + 1) & 1], bhi[(it + 1) & 1]);
+            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
+            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
+            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
+            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l1, acc[it][1], 0, 0, 0);
+            // next step's x operands, one or two eighths per iteration
+#pragma unroll
+            for (int e = it * 8 / NT; e < (it + 1) * 8 / NT; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
+            if (it < 2) load_x(rsx, s3, it);
+            if (it >= 2 && it < 2 + NTW) load_B(rsB, s3, wave * NTW + (it - 2));
+            if (s == 1 && it == NT - 1) mnext = load_meta(c + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (s == SPC / 2) put_weights(c + 1, (ws + 1) % 3, mnext);
+    };
+
+    for (int c = 0; c < C; ++c) {
+        const int ws = c % 3;
+        step(c, std::integral_constant<int, 0>{}, ws, fA, fB);
+        step(c, std::integral_constant<int, 1>{}, ws, fB, fA);
+        step(c, std::integral_constant<int, 2>{}, ws, fA, fB);
+        step(c, std::integral_constant<int, 3>{}, ws, fB, fA);
+        if constexpr (SPC == 8) {
+            step(c, std::integral_constant<int, 4>{}, ws, fA, fB);
+            step(c, std::integral_constant<int, 5>{}, ws, fB, fA);
+            step(c, std::integral_constant<int, 6>{}, ws, fA, fB);
+            step(c, std::integral_constant<int, 7>{}, ws, fB, fA);
+        }
+        mcur = mnext;
+        rsx0 = rsx1; rsB0 = rsB1;
+        rsx1 = chunk_rsrc(xrow, xrb, c + 2);
+        rsB1 = chunk_rsrc(Brow, Brb, c + 2);
+    }
+    store_state(make_rsrc(p.fin + b * p.sf_b + h * p.sf_h, slice_fin * 4), DT_F32, (int)p.sf_p);
+}
+
+static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
+
+}  // namespace quad
+
+// The four-tiles-per-workgroup kernel serves the fused call without a `states` output, for bf16 x / B with 16-byte
+// aligned rows, unit-stride dt / dA_cumsum rows, and head counts that put four tiles of one group in a workgroup.
+bool quad_supported(const Params &p)
+{
+    using quad::aligned;
+    if (p.states || !p.out || !p.fin) return false;
+    if (p.dt_in != DT_BF16) return false;
+    if (p.headdim % 32 != 0) return false;
+    if (p.dstate != 64 && p.dstate != 128) return false;
+    if (p.Q != 128 && p.Q != 256) return false;
+    if (((p.nheads / p.ngroups) * (p.headdim / 32)) % 4 != 0) return false;      // 4 tiles of one (batch, group)
+    if (!aligned(p.x, 16) || (p.sx_b | p.sx_l | p.sx_h) % 8) return false;
+    if (!aligned(p.B, 16) || (p.sB_b | p.sB_l | p.sB_g) % 8) return false;
+    if ((int64_t)p.Q * 2 * p.sx_l >= (1LL << 31) || (int64_t)p.Q * 2 * p.sB_l >= (1LL << 31)) return false;
+    if (p.sdt_k != 1 || p.sda_k != 1) return false;
+    if (!aligned(p.dt, 16) || (p.sdt_b | p.sdt_h | p.sdt_c) % 4) return false;
+    if (!aligned(p.dacs, 16) || (p.sda_b | p.sda_h | p.sda_c) % 4) return false;
+    if (!aligned(p.out, 16) || (p.so_b | p.so_c | p.so_h | p.so_p) % 4) return false;
+    if (!aligned(p.fin, 16) || (p.sf_b | p.sf_h | p.sf_p) % 4) return false;
+    if (p.init && (!aligned(p.init, 16) || (p.sin_b | p.sin_h | p.sin_p) % 4)) return false;
+    if ((int64_t)p.headdim * p.so_p >= (1LL << 28) || (int64_t)p.headdim * p.sf_p >= (1LL << 28)) return false;
+    return true;
+}
+
+template <int NT, int SPC, bool SEQ, bool F32IO>
+static hipError_t launch_quad_k(const Params &p, dim3 grid, hipStream_t s)
+{
+    constexpr int lds = quad::lds_bytes<NT, SPC>();
+    static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
+    if (lds > 65536 && !configured) {
+        hipError_t e = hipFuncSetAttribute((const void *)quad::quad_kernel<NT, SPC, SEQ, F32IO>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL((quad::quad_kernel<NT, SPC, SEQ, F32IO>), grid, dim3(256), lds, s, p);
+    return hipGetLastError();
+}
+
+template <int NT, int SPC>
+static hipError_t launch_quad_t(const Params &p, hipStream_t s)
+{
+    dim3 grid((((p.n_items >> 2) + 7) / 8) * 8);
+    const bool f32io = p.dt_out == DT_F32 && (!p.init || p.dt_init == DT_F32);
+    if (p.seq) return f32io ? launch_quad_k<NT, SPC, true, true>(p, grid, s) : launch_quad_k<NT, SPC, true, false>(p, grid, s);
+    return f32io ? launch_quad_k<NT, SPC, false, true>(p, grid, s) : launch_quad_k<NT, SPC, false, false>(p, grid, s);
+}
+
+hipError_t launch_quad(const Params &p_in, hipStream_t s)
+{
+    Params p = p_in;
+    p.n_items = p.batch * p.nheads * (p.headdim / 32);
+    if (p.n_items <= 0) return hipSuccess;
+    const int nt = p.dstate / 16, spc = p.Q / 32;
+    if (nt == 8 && spc == 8) return launch_quad_t<8, 8>(p, s);
+    if (nt == 8 && spc == 4) return launch_quad_t<8, 4>(p, s);
+    if (nt == 4 && spc == 8) return launch_quad_t<4, 8>(p, s);
+    return launch_quad_t<4, 4>(p, s);
+}
+
+}  // namespace ssd
