@@ -129,10 +129,12 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
                          int dt_softplus, float dt_min, float dt_max, void *stream);
 
 /*
- * Tuning / test hook with no counterpart in the reference: how many waves split the tokens of a chunk in the bf16
- * MFMA kernels.  0 = let the library choose from the problem size (the default), 2 or 4 = force that split for
- * every later call of this process.  Returns the previous setting, or SSD_ERR_SHAPE for any other value.
- * Results agree between the settings to rounding (the tokens are summed in another order), not bit for bit.
+ * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
+ * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
+ * waves per state tile; 1 = one wave per state tile (the fused kernel with four tiles per workgroup) wherever that
+ * kernel applies.  The setting holds for every later call of this process.  Returns the previous setting, or
+ * SSD_ERR_SHAPE for any other value.  Results agree between the settings to rounding (the tokens are summed in
+ * another order), not bit for bit.
  */
 int ssd_set_token_split(int waves);
 

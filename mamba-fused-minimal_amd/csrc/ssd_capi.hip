@@ -10,7 +10,7 @@ namespace {
 using ssd::Params;
 using ssd::PassParams;
 
-int g_forced_split = 0;     // ssd_set_token_split: a forced split also forces the token-split kernels
+int g_forced_split = 0;     // ssd_set_token_split: 0 = choose, 1 = four-tile kernel, 2 / 4 = token-split kernels
 
 bool dtype_ok(int dt) { return dt == SSD_F32 || dt == SSD_BF16 || dt == SSD_F16; }
 
@@ -84,7 +84,8 @@ int run(const Params &p, bool fused, void *stream)
     // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
     // kernel, which puts four waves on every tile, has the shorter chunk.
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
-    if (fused && g_forced_split == 0 && tiles >= 512 && ssd::quad_supported(p)) e = ssd::launch_quad(p, s);
+    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
+        e = ssd::launch_quad(p, s);
     else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
     return (int)e;
 }
@@ -226,9 +227,11 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
 
 int ssd_set_token_split(int waves)
 {
-    if (waves != 0 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;
+    if (waves != 0 && waves != 1 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;
+    const int old = g_forced_split;
     g_forced_split = waves;
-    return ssd::set_token_split(waves);
+    ssd::set_token_split(waves == 1 ? 0 : waves);
+    return old;
 }
 
 }  // extern "C"

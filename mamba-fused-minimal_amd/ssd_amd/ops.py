@@ -176,9 +176,10 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
 
 
 def set_token_split(waves):
-    """Tuning / test hook (no counterpart in the reference): force how many waves split the tokens of a chunk in
-    the bf16 MFMA kernels (2 or 4), or 0 to let the library choose.  Returns the previous setting."""
+    """Tuning / test hook (no counterpart in the reference): 2 or 4 = the token-split bf16 MFMA kernels with that
+    many waves per state tile, 1 = the fused kernel with one wave per tile and four tiles per workgroup wherever it
+    applies, 0 = let the library choose.  Returns the previous setting."""
     rc = _lib.load().ssd_set_token_split(int(waves))
     if rc < 0:
-        raise ValueError("token split must be 0, 2 or 4")
+        raise ValueError("token split must be 0, 1, 2 or 4")
     return rc

@@ -70,7 +70,7 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 256, 2, 0, 0, 0.0, 1.0, None) == -2
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o.bfloat16()), T(o), 1, 256, 2, 256, 0, 0.0, 1.0, None) == -3
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 4096, 2, 2048, 0, 0.0, 1.0, None) == -2   # chunk > 1024
-    assert lib.ssd_set_token_split(3) == -2 and lib.ssd_set_token_split(0) == 0
+    assert lib.ssd_set_token_split(3) == -2 and lib.ssd_set_token_split(1) == 0 and lib.ssd_set_token_split(0) == 1
 
 
 def test_signatures_match_reference_call_surface():
