@@ -87,10 +87,14 @@ __device__ __forceinline__ void store4(__amdgpu_buffer_rsrc_t rs, int dt, int vo
 
 struct Frag { uint32_t hi[2][4], lo[2][4]; };
 
-constexpr int kRing = 4;            // steps of B kept in LDS (requested three steps ahead)
+// Steps of B and x kept in LDS (requested ring - 1 steps ahead, into the next chunk at most).  A ring of 8 was
+// measured too (chunk 256 only): same time, so the requests are not what the kernel waits for.
+constexpr int kRingSteps = 4;
+template <int SPC> constexpr int ring_of() { return kRingSteps <= SPC ? kRingSteps : 4; }
 
-template <int NT, int SPC> constexpr int wave_lds() { return 4 * 2048 + 3 * 32 * SPC * 4; }     // x ring + weights
-template <int NT, int SPC> constexpr int lds_bytes() { return kRing * NT * 1024 + 4 * wave_lds<NT, SPC>(); }
+template <int NT, int SPC> constexpr int wave_lds() { return ring_of<SPC>() * 2048 + 3 * 32 * SPC * 4; }     // x ring + weights
+constexpr int kStage = 1024;        // per wave: one 16 x 16 fp32 block of the state on its way to memory
+template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * NT * 1024 + 4 * (wave_lds<NT, SPC>() + kStage); }
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (chunk_size / 32: 4 or 8);
 // F32IO = out and initial states are fp32 (or the latter absent): element-type branches fold away.
@@ -98,14 +102,16 @@ template <int NT, int SPC, bool HAS_SEQ, bool F32IO>
 __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
 {
     constexpr int Q = 32 * SPC;
+    constexpr int kRing = ring_of<SPC>(), kDist = kRing - 1;
     constexpr int TPL = Q / 64;         // tokens per lane when the chunk's weights are computed (2 or 4)
     constexpr int NTW = NT / 4;         // B tile blocks (32 tokens x 16 columns, 1 KB) a wave fetches per step
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     char *bring = lds;                                                   // kRing x NT blocks of 1 KB, shared
-    char *xring = lds + kRing * NT * 1024 + wave * wave_lds<NT, SPC>();  // 4 slots x (32 tokens x 64 bytes)
-    char *wbuf = xring + 4 * 2048;                                       // 3 slots x Q weights
+    char *xring = lds + kRing * NT * 1024 + wave * wave_lds<NT, SPC>();  // kRing slots x (32 tokens x 64 bytes)
+    char *wbuf = xring + kRing * 2048;                                   // 3 slots x Q weights
+    char *stage = lds + kRing * NT * 1024 + 4 * wave_lds<NT, SPC>() + wave * kStage;
 
     // Work item -> (batch, head, row slice); the four items of a workgroup share batch and group (checked on the
     // host).  Consecutive workgroups sit on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so a
@@ -172,10 +178,11 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
 #endif
     };
 #pragma clang diagnostic pop
-    // results of read_Bt become valid here (and every other LDS operation of the wave is complete)
-    auto wait_Bt = [&](u32x2 &lo, u32x2 &hi) {
+    // The results of a read_Bt become valid here.  LDS operations complete in order, so the pair has arrived once
+    // no more LDS operations are outstanding than were issued after it: nc = that number, at least.
+    auto wait_Bt = [&](auto nc, u32x2 &lo, u32x2 &hi) {
 #if defined(__HIP_DEVICE_COMPILE__)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi) : : "memory");
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(decltype(nc)::value) : "memory");
 #else
         (void)lo; (void)hi;
 #endif
@@ -187,7 +194,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     auto load_x = [&](__amdgpu_buffer_rsrc_t rs, int s, int i) {
 #if defined(__HIP_DEVICE_COMPILE__)
         typedef __attribute__((address_space(3))) void *lds_ptr;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xring + (s & 3) * 2048 + i * 1024), 16, xlane,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xring + (s % kRing) * 2048 + i * 1024), 16, xlane,
                                                  (int)((32 * s + 4 * i) * xrb), 0, 0);
 #else
         (void)rs; (void)s; (void)i; (void)xlane;
@@ -241,7 +248,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     auto read_operands = [&](int s, int ws, uint32_t (&xr)[8], float (&wv)[8]) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            xr[j] = *(const uint32_t *)(xring + (s & 3) * 2048 + xst_rd + 1024 * (j >> 2) + 256 * (j & 3));
+            xr[j] = *(const uint32_t *)(xring + (s % kRing) * 2048 + xst_rd + 1024 * (j >> 2) + 256 * (j & 3));
         const f32x4 wlo = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg));
         const f32x4 whi = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg + 4));
         wv[0] = wlo.x; wv[1] = wlo.y; wv[2] = wlo.z; wv[3] = wlo.w;
@@ -265,11 +272,30 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     const int64_t slice_out = (int64_t)(p.headdim - 1) * p.so_p + p.dstate;
     const int64_t slice_fin = (int64_t)(p.headdim - 1) * p.sf_p + p.dstate;
     auto store_state = [&](__amdgpu_buffer_rsrc_t rs, int dt, int row_pitch) {
-        const int voff = (p0 + 2 * i16) * row_pitch + 4 * kg;
+        // The accumulators hold a 16 x 16 block as (lane%16 = row, lane/16 = group of four columns): neighbouring
+        // lanes sit in different rows, 512 bytes apart, and the memory pipeline, which merges only what adjacent
+        // lanes address, would take every lane's 16 bytes as a request of its own (measured: 64 cycles of the
+        // compute unit's store path per instruction instead of 16).  So each block passes through 1 KB of LDS and
+        // comes back as (lane/4 = row, lane%4 = group): four adjacent lanes then write 64 contiguous bytes.  The
+        // column group is XORed with row/4 in LDS, which keeps both the 16-byte writes and reads off shared banks.
+        const int voff = (p0 + 2 * (lane >> 2)) * row_pitch + 4 * (lane & 3);
+        f32x4 *wr = (f32x4 *)(stage + i16 * 64 + ((kg ^ (i16 >> 2)) << 4));
+        const f32x4 *rd = (const f32x4 *)(stage + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4));
+        // LDS operations of one wave execute in order, so block k + 1 may be written right behind the read of
+        // block k; the store of a block follows kLag blocks later, when its read has long returned
+        constexpr int kLag = 4;
+        f32x4 v[2 * NT];
 #pragma unroll
-        for (int it = 0; it < NT; ++it)
-#pragma unroll
-            for (int jp = 0; jp < 2; ++jp) store4(rs, dt, voff, jp * row_pitch + 16 * it, acc[it][jp]);
+        for (int k = 0; k < 2 * NT + kLag; ++k) {
+            if (k < 2 * NT) {
+                *wr = acc[k >> 1][k & 1];
+                v[k] = *rd;
+            }
+            if (k >= kLag) {
+                const int j = k - kLag;
+                store4(rs, dt, voff, (j & 1) * row_pitch + 16 * (j >> 1), v[j]);
+            }
+        }
     };
 #pragma unroll
     for (int it = 0; it < NT; ++it)
@@ -293,7 +319,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     // ---- prologue: rows past the end of the sequence are not fetched and leave their LDS slots untouched; their
     // weight is zero, so the slots only have to hold finite numbers.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *(u32x4 *)(xring + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+    for (int i = 0; i < 2 * kRing; ++i) *(u32x4 *)(xring + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
     for (int i = 0; i < kRing * NTW; ++i)
         *(u32x4 *)(bring + (i * 4 + wave) * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
@@ -302,9 +328,9 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     Meta mcur = load_meta(0);
     __amdgpu_buffer_rsrc_t rsx0 = chunk_rsrc(xrow, xrb, 0), rsx1 = chunk_rsrc(xrow, xrb, 1);
     __amdgpu_buffer_rsrc_t rsB0 = chunk_rsrc(Brow, Brb, 0), rsB1 = chunk_rsrc(Brow, Brb, 1);
-    // requests of the steps 0..2, in the order (x, x, B...) that every later step keeps
+    // requests of the steps 0..kDist-1, in the order (x, x, B...) that every later step keeps
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
+    for (int s = 0; s < kDist; ++s) {
         load_x(rsx0, s, 0); load_x(rsx0, s, 1);
 #pragma unroll
         for (int k = 0; k < NTW; ++k) load_B(rsB0, s, wave * NTW + k);
@@ -312,30 +338,43 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     }
     put_weights(0, 0, mcur);
     Frag fA, fB;
+    // B operands (transposed blocks) travel kAhead iterations ahead of the MFMAs that use them, across step
+    // boundaries: block t of the stream of (step, tile) pairs sits in slot t % 4.  An LDS read takes longer than the
+    // four MFMAs of one iteration, so a single block in flight would leave the matrix pipe waiting every iteration.
+    constexpr int kAhead = 3;
+    static_assert(NT % 4 == 0 && kAhead < 4 && kAhead <= NT, "slot of a block = its tile index % 4");
+    constexpr int kStores = 2 * NT;     // vector-memory operations of one store_state
+    u32x2 blo[4], bhi[4];
     {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * (2 + NTW) - 2));      // the two x requests of step 0
+        // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 1) * (2 + NTW)));
+        __builtin_amdgcn_s_barrier();   // ... and every other wave's blocks of step 0
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
         read_operands(0, 0, xr, wv);
 #pragma unroll
         for (int q = 0; q < 4; ++q) { frag_piece(q, 0, xr, wv, fA); frag_piece(q, 1, xr, wv, fA); }
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<kAhead>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            read_Bt(std::integral_constant<int, i * 1024>{}, blo[i], bhi[i]);
+        });
+        __builtin_amdgcn_sched_barrier(0);
     }
     int32_t prev_id = 0;
     Meta mnext = mcur;
 
     // One 32-token step s of chunk c (weight slot ws): fc = x operands of this step, fn receives those of step + 1.
+    // Vector-memory requests of a step, in program order: [the state stores, step 0 only], the two x requests of
+    // step + 3 (iteration 0), this wave's B requests of step + 3 (after the barrier in iteration NT - kAhead).
+    // Memory operations complete in order and the compiler does not track loads that write LDS, so the waits for
+    // them are explicit: "no more outstanding than were issued after the one needed".
     auto step = [&](int c, auto sc, int ws, Frag &fc, Frag &fn) {
         constexpr int s = decltype(sc)::value;
-        // This step needs its B tile (every wave's part of it) and, for the next step's operands, this wave's x
-        // rows of step + 1.  A step issues its vector-memory requests in the order x, x, B.. (three steps ahead);
-        // memory operations complete in order, so this wave's B part (requested three steps ago) and the x rows of
-        // step + 1 (two steps ago) have landed once no more than the NTW B requests of that step and the 2 + NTW
-        // requests of the step in between are outstanding.  The compiler does not track loads that write LDS, so
-        // the wait is explicit; the barrier then publishes every wave's part and tells that all waves are done
-        // reading the tile of the previous step, whose ring slot this step's requests overwrite.
-        constexpr int kAfter = NTW + (2 + NTW);
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kAfter));
-        __builtin_amdgcn_s_barrier();
+        // x rows of step + 1 (this wave's own, requested two steps ago): behind them came the B requests of that
+        // step and all requests of the steps s + 2 - kDist .. s - 1 (with the state stores, if step 0 is among them)
+        constexpr bool st_top = s >= 1 && s <= kDist - 2;         // step 0 among them
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(NTW + (kDist - 2) * (2 + NTW) + (st_top ? kStores : 0)));
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
         if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
@@ -356,22 +395,35 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
                 for (int jp = 0; jp < 2; ++jp) acc[it][jp] *= sc;
         }
         // requests of this step: x rows and this wave's B blocks of step + 3 (this chunk or the next)
-        const auto rsB = s + 3 < SPC ? rsB0 : rsB1;
-        const auto rsx = s + 3 < SPC ? rsx0 : rsx1;
-        const int s3 = (s + 3) % SPC;
+        const auto rsB = s + kDist < SPC ? rsB0 : rsB1;
+        const auto rsx = s + kDist < SPC ? rsx0 : rsx1;
+        const int s3 = (s + kDist) % SPC;
         const bf16x8 h0 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[0][0], fc.hi[0][1], fc.hi[0][2], fc.hi[0][3]});
         const bf16x8 h1 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[1][0], fc.hi[1][1], fc.hi[1][2], fc.hi[1][3]});
         const bf16x8 l0 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[0][0], fc.lo[0][1], fc.lo[0][2], fc.lo[0][3]});
         const bf16x8 l1 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[1][0], fc.lo[1][1], fc.lo[1][2], fc.lo[1][3]});
-        u32x2 blo[2], bhi[2];            // B operand of tile it in slot it % 2, the next one in flight in the other
-        read_Bt(std::integral_constant<int, ((s % kRing) * NT) * 1024>{}, blo[0], bhi[0]);
-        __builtin_amdgcn_sched_barrier(0);   // operand reads above, the requests that reuse their slots below
+        __builtin_amdgcn_sched_barrier(0);   // stores and operand reads above, the requests of this step below
         static_for<NT>([&](auto itc) {
             constexpr int it = decltype(itc)::value;
-            wait_Bt(blo[it & 1], bhi[it & 1]);
-            const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it & 1].x, blo[it & 1].y, bhi[it & 1].x, bhi[it & 1].y});
-            if constexpr (it + 1 < NT)
-                read_Bt(std::integral_constant<int, ((s % kRing) * NT + it + 1) * 1024>{}, blo[(it + 1) & 1], bhi[(it + 1) & 1]);
+            // the kAhead - 1 blocks behind this one (two reads each) may still be in flight
+            wait_Bt(std::integral_constant<int, 2 * (kAhead - 1)>{}, blo[it % 4], bhi[it % 4]);
+            const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it % 4].x, blo[it % 4].y, bhi[it % 4].x, bhi[it % 4].y});
+            if constexpr (it == NT - kAhead) {
+                // The next read is the first of step + 1's tile: this wave's blocks of it (requested three steps
+                // ago) have landed once only the requests of step - 1 and the x requests of this step (with the
+                // stores, if either was step 0) are outstanding; the barrier publishes every wave's blocks.  It
+                // also tells that all waves are through with the tile of step - 1, whose ring slot the B requests
+                // below overwrite.
+                constexpr bool st_mid = s < kDist - 1;       // step 0 among the steps s + 2 - kDist .. s
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 2) * (2 + NTW) + 2 + (st_mid ? kStores : 0)));
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+            {
+                constexpr int tn = it + kAhead;     // block kAhead iterations on: this step's tile or the next one's
+                constexpr int blk = tn < NT ? (s % kRing) * NT + tn : ((s + 1) % kRing) * NT + tn - NT;
+                read_Bt(std::integral_constant<int, blk * 1024>{}, blo[tn % 4], bhi[tn % 4]);
+            }
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
@@ -379,8 +431,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
             // next step's x operands, one or two eighths per iteration
 #pragma unroll
             for (int e = it * 8 / NT; e < (it + 1) * 8 / NT; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
-            if (it < 2) load_x(rsx, s3, it);
-            if (it >= 2 && it < 2 + NTW) load_B(rsB, s3, wave * NTW + (it - 2));
+            if (it == 0) { load_x(rsx, s3, 0); load_x(rsx, s3, 1); }
+            if (it >= NT - kAhead && it < NT - kAhead + NTW) load_B(rsB, s3, wave * NTW + (it - (NT - kAhead)));
             if (s == 1 && it == NT - 1) mnext = load_meta(c + 1);
             __builtin_amdgcn_sched_barrier(0);
         });
