@@ -129,6 +129,22 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
                          int dt_softplus, float dt_min, float dt_max, void *stream);
 
 /*
+ * The consumer of the passed states: the state-dependent half of the chunk scan.  Replaces that part of
+ * _chunk_scan_fwd_kernel (kernels/ssd_chunk_scan.py:94-117; wrapper _chunk_scan_fwd, :172-224):
+ *   y[b,cQ+m,h,p] = scale_m * sum_n C[b,cQ+m,h/(H/G),n] * prev_states[b,c,h,p,n],
+ *   scale_m = exp(dA_cumsum[b,h,c,m]) * [seq_idx[b,cQ+m] == seq_idx[b,cQ-1]]  (the latter taken as 0 when c == 0).
+ * C: (batch, seqlen, ngroups, dstate); prev_states: (batch, nchunks, nheads, headdim, dstate), the `out` of the
+ * state passing / fused calls above; dA_cumsum as above; seq_idx nullable; y: (batch, seqlen, nheads, headdim),
+ * f32/bf16/f16.  Innermost strides of C, prev_states and y must be 1.  accumulate != 0 adds to what y holds (the
+ * intra-chunk half of the scan computed elsewhere) instead of overwriting it.  bf16 C with fp32 states, dstate
+ * 64/128, chunk size 64/128/256 and headdim % 32 == 0 run on the matrix cores with the fp32 state entering as
+ * bf16 hi + lo (the reference rounds the state to C's element type); everything else on a plain FMA kernel.
+ */
+int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states, const ssd_tensor *dA_cumsum,
+                              const ssd_tensor *seq_idx, const ssd_tensor *y, const ssd_dims *dims, int accumulate,
+                              void *stream);
+
+/*
  * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
  * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
  * waves per state tile; 1 = one wave per state tile (the fused kernel with four tiles per workgroup) wherever that

@@ -225,6 +225,42 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
     return (int)ssd::launch_chunk_cumsum(p, (hipStream_t)stream);
 }
 
+int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states, const ssd_tensor *dA_cumsum,
+                              const ssd_tensor *seq_idx, const ssd_tensor *y, const ssd_dims *dims, int accumulate,
+                              void *stream)
+{
+    if (!present(C) || !present(prev_states) || !present(dA_cumsum) || !present(y) || !dims) return SSD_ERR_NULL;
+    const ssd_dims &d = *dims;
+    if (d.batch <= 0 || d.seqlen <= 0 || d.nheads <= 0 || d.headdim <= 0 || d.dstate <= 0 || d.ngroups <= 0 ||
+        d.chunk_size <= 0 || d.nheads % d.ngroups != 0 || d.nchunks != (d.seqlen + d.chunk_size - 1) / d.chunk_size)
+        return SSD_ERR_SHAPE;
+    if (!dtype_ok(C->dtype) || !dtype_ok(prev_states->dtype) || !dtype_ok(y->dtype) || dA_cumsum->dtype != SSD_F32)
+        return SSD_ERR_DTYPE;
+    if (C->stride[3] != 1 || prev_states->stride[4] != 1 || y->stride[3] != 1) return SSD_ERR_STRIDE;
+    ssd::ScanParams p;
+    memset(&p, 0, sizeof(p));
+    p.Cm = C->data; p.dt_C = C->dtype;
+    p.sC_b = C->stride[0]; p.sC_l = C->stride[1]; p.sC_g = C->stride[2];
+    p.states = prev_states->data; p.dt_states = prev_states->dtype;
+    p.sst_b = prev_states->stride[0]; p.sst_c = prev_states->stride[1]; p.sst_h = prev_states->stride[2];
+    p.sst_p = prev_states->stride[3];
+    p.dacs = (const float *)dA_cumsum->data;
+    p.sda_b = dA_cumsum->stride[0]; p.sda_h = dA_cumsum->stride[1]; p.sda_c = dA_cumsum->stride[2];
+    p.sda_k = dA_cumsum->stride[3];
+    if (present(seq_idx)) {
+        p.seq = (const int32_t *)seq_idx->data;
+        p.ssq_b = seq_idx->stride[0]; p.ssq_l = seq_idx->stride[1];
+    }
+    p.out = y->data; p.dt_out = y->dtype;
+    p.so_b = y->stride[0]; p.so_l = y->stride[1]; p.so_h = y->stride[2];
+    p.batch = d.batch; p.seqlen = d.seqlen; p.nheads = d.nheads; p.headdim = d.headdim; p.dstate = d.dstate;
+    p.ngroups = d.ngroups; p.Q = d.chunk_size; p.C = d.nchunks;
+    p.accumulate = accumulate ? 1 : 0;
+    int rc = check_device();
+    if (rc) return rc;
+    return (int)ssd::launch_scan_states(p, (hipStream_t)stream);
+}
+
 int ssd_set_token_split(int waves)
 {
     if (waves != 0 && waves != 1 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;

@@ -68,6 +68,23 @@ struct CumsumParams {
     float dt_min, dt_max;
 };
 
+// State-consuming half of the chunk scan: y = scale * (C . prev_states).
+struct ScanParams {
+    const void *Cm;        // (b, L, G, N)
+    const void *states;    // (b, C, H, P, N): the state entering each chunk
+    const float *dacs;     // (b, H, C, Q)
+    const int32_t *seq;    // (b, L) or null
+    void *out;             // (b, L, H, P)
+    int batch, seqlen, nheads, headdim, dstate, ngroups, Q, C;
+    int64_t sC_b, sC_l, sC_g;
+    int64_t sst_b, sst_c, sst_h, sst_p;
+    int64_t sda_b, sda_h, sda_c, sda_k;
+    int64_t ssq_b, ssq_l;
+    int64_t so_b, so_l, so_h;
+    int dt_C, dt_states, dt_out;
+    int accumulate;        // add to what out holds instead of overwriting it
+};
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t hbits) { return __builtin_bit_cast(float, hbits << 16); }
 
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
@@ -98,6 +115,8 @@ hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state
 bool quad_supported(const Params &p);
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
+hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);
+bool scan_states_mfma_supported(const ScanParams &p);
 int set_token_split(int wv);      // 0 = automatic; 2 or 4 forces the token split of the MFMA kernels; returns the old value
 
 }  // namespace ssd

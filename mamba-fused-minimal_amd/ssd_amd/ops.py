@@ -175,6 +175,47 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
     return dA_cumsum, dt_out
 
 
+def _chunk_scan_states_fwd(C, prev_states, dA_cumsum, seq_idx=None, out=None, out_dtype=None, accumulate=False):
+    """The state-consuming half of the reference's ``_chunk_scan_fwd`` (kernels/ssd_chunk_scan.py:94-117, wrapper
+    :172-224): y[b,cQ+m,h,:] = scale_m * (C[b,cQ+m,g,:] . prev_states[b,c,h]), scale_m = exp(dA_cumsum[b,h,c,m]) where
+    seq_idx[b,cQ+m] equals seq_idx[b,cQ-1] (0 for the first chunk) and 0 elsewhere.
+
+    C (batch, seqlen, ngroups, dstate); prev_states (batch, nchunks, nheads, headdim, dstate), the ``out`` of the
+    state passing; dA_cumsum (batch, nheads, nchunks, chunk_size).  Returns y (batch, seqlen, nheads, headdim) of
+    ``out_dtype`` (default: C's, as the reference's ``out`` takes x's); with ``out=`` the result goes there, and with
+    ``accumulate=True`` it is added to what ``out`` holds (the intra-chunk half of the scan)."""
+    batch, seqlen, ngroups, dstate = C.shape
+    _, nchunks, nheads, headdim, _ = prev_states.shape
+    chunk_size = dA_cumsum.shape[-1]
+    assert nheads % ngroups == 0
+    assert prev_states.shape == (batch, nchunks, nheads, headdim, dstate)
+    assert dA_cumsum.shape == (batch, nheads, nchunks, chunk_size)
+    assert nchunks == math.ceil(seqlen / chunk_size)
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+        if seq_idx.dtype != torch.int32:
+            seq_idx = seq_idx.to(torch.int32)
+    _lib.require_device(C, "_chunk_scan_states_fwd")
+    if out is None:
+        assert not accumulate, "accumulate=True needs the tensor to add to (out=)"
+        out = torch.empty(batch, seqlen, nheads, headdim, device=C.device, dtype=out_dtype or C.dtype)
+    else:
+        assert out.shape == (batch, seqlen, nheads, headdim) and out.stride(-1) == 1
+    if C.stride(-1) != 1:
+        C = C.contiguous()
+    if prev_states.stride(-1) != 1:
+        prev_states = prev_states.contiguous()
+    if dA_cumsum.dtype != torch.float32:
+        dA_cumsum = dA_cumsum.float()
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    with torch.cuda.device(C.device):
+        rc = _lib.load().ssd_chunk_scan_states_fwd(_lib.tensor_arg(C), _lib.tensor_arg(prev_states),
+                                                   _lib.tensor_arg(dA_cumsum), _lib.tensor_arg(seq_idx),
+                                                   _lib.tensor_arg(out), dims, int(bool(accumulate)), _stream(C))
+    _lib.check(rc, "ssd_chunk_scan_states_fwd")
+    return out
+
+
 def set_token_split(waves):
     """Tuning / test hook (no counterpart in the reference): 2 or 4 = the token-split bf16 MFMA kernels with that
     many waves per state tile, 1 = the fused kernel with one wave per tile and four tiles per workgroup wherever it

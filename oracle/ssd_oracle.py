@@ -20,6 +20,7 @@ fused_ref              kernels/fused_globalbar.py:201-266, kernels/fused_concurr
                        (same contract: chunk state followed by state passing)
 bmm_chunk_ref          kernels/ssd_bmm.py:31-134   (the step before the chunk scan; outside the path, used to
 chunk_scan_ref         kernels/ssd_chunk_scan.py:38-215   run the path inside a whole SSD forward, main.py:60-104)
+chunk_scan_states_ref  kernels/ssd_chunk_scan.py:94-117   (the state-consuming half of the chunk scan alone)
 token_scan_ref         no counterpart in the reference: token-serial y_t = C_t . h_t + D x_t in fp64, which pins
                        the chunked composition cumsum -> chunk state -> state passing -> bmm -> chunk scan.
 token_recurrence_ref   no counterpart in the reference: an independent, chunk-free
@@ -303,6 +304,27 @@ def chunk_scan_ref(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=None
         return y, None
     zf = z.float()
     return y * zf * torch.sigmoid(zf), y
+
+
+def chunk_scan_states_ref(C, states, dA_cumsum, seq_idx=None):
+    """Follows kernels/ssd_chunk_scan.py:94-117 alone: the contribution of the state entering each chunk,
+    y[b, cQ+m, h, :] = scale_m * (C[b, cQ+m, g, :] . states[b, c, h]),  scale_m = exp(dA_cumsum[b, h, c, m]) where
+    seq_idx[b, cQ+m] == seq_idx[b, cQ-1] (taken as 0 for c == 0), else 0.  fp32 throughout: the reference's rounding
+    of the states to C's element type (:110) is not restated.  Returns y (batch, seqlen, nheads, headdim) fp32."""
+    batch, seqlen, ngroups, dstate = C.shape
+    _, nchunks, nheads, headdim, _ = states.shape
+    Q = dA_cumsum.shape[-1]
+    ratio = nheads // ngroups
+    y = torch.zeros(batch, seqlen, nheads, headdim, dtype=torch.float32)
+    for c in range(nchunks):
+        lo, hi = c * Q, min((c + 1) * Q, seqlen)
+        Cc = C[:, lo:hi].float().repeat_interleave(ratio, dim=2)                      # (b, m, H, N)
+        scale = torch.exp(dA_cumsum[:, :, c, :hi - lo].float()).permute(0, 2, 1)      # (b, m, H)
+        if seq_idx is not None:
+            prev = seq_idx[:, lo - 1].long() if c >= 1 else torch.zeros(batch, dtype=torch.long)
+            scale = scale * (seq_idx[:, lo:hi].long() == prev[:, None]).float()[:, :, None]
+        y[:, lo:hi] = torch.einsum("bmhn,bhpn->bmhp", Cc, states[:, c].float()) * scale[..., None]
+    return y
 
 
 def token_scan_ref(x, B, C, dt_tok, A, D=None, initial_states=None, seq_idx=None):

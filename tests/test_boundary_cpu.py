@@ -70,6 +70,15 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 256, 2, 0, 0, 0.0, 1.0, None) == -2
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o.bfloat16()), T(o), 1, 256, 2, 256, 0, 0.0, 1.0, None) == -3
     assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 4096, 2, 2048, 0, 0.0, 1.0, None) == -2   # chunk > 1024
+    # scan consumer: same order of checks (null, shape, dtype, stride) before any device work
+    Cm = torch.zeros(1, 256, 1, 128, dtype=torch.bfloat16)
+    st = torch.zeros(1, 1, 2, 64, 128)
+    dA = torch.zeros(1, 2, 1, 256)
+    y = torch.zeros(1, 256, 2, 64)
+    assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(None), T(dA), T(None), T(y), dims, 0, None) == -1
+    assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA), T(None), T(y), bad, 0, None) == -2
+    assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA.bfloat16()), T(None), T(y), dims, 0, None) == -3
+    assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA), T(None), T(y.transpose(2, 3)), dims, 0, None) == -4
     assert lib.ssd_set_token_split(3) == -2 and lib.ssd_set_token_split(1) == 0 and lib.ssd_set_token_split(0) == 1
 
 

@@ -299,6 +299,62 @@ def test_chunk_cumsum_strided_dt_and_pipeline(ops, oracle):
     _check("pipeline.final", fin, want_fin)
 
 
+# ------------------------------------------------------------------ the consumer of the passed states
+@pytest.mark.parametrize("kw", [
+    dict(),                                              # chunk 256, dstate 128, headdim 64: matrix-core kernel
+    dict(L=1000, nseq=5),                                # ragged last chunk + packed sequences
+    dict(Q=128, L=1024, H=8, G=4),                       # chunk 128, grouped C
+    dict(Q=64, L=512, N=64),                             # chunk 64, dstate 64
+    dict(P=32, H=4),                                     # headdim 32: two row blocks per item
+    dict(P=128, H=4),                                    # headdim 128: two items per head
+    dict(L=300, H=3, P=40, N=24, G=1, Q=64),             # nothing aligned: plain FMA kernel
+    dict(dtype="fp16"),                                  # fp16 C: plain FMA kernel
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
+def test_chunk_scan_states(ops, oracle, kw):
+    base = dict(b=2, L=1024, H=6, G=1, init=True)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    C, seq, dA = d["C"], d["seq_idx"], d["dA_cumsum"]
+    prev, _ = oracle.fused_ref(d["B"], d["x"], d["dt"], dA, initial_states=d["initial_states"], seq_idx=seq)
+    want = oracle.chunk_scan_states_ref(C, prev, dA, seq_idx=seq)
+    Cd, pd, dAd, sd = _dev(C), _dev(prev), _dev(dA), _dev(seq)
+    print(f"[scan_states] C{tuple(C.shape)} {C.dtype} states{tuple(prev.shape)}", flush=True)
+    y = ops._chunk_scan_states_fwd(Cd, pd, dAd, seq_idx=sd, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert y.dtype == torch.float32 and y.shape == want.shape
+    _check("scan_states.f32", y, want)
+    # default output type follows C (the reference's out follows x); judged at the reference's own tolerance
+    yb = ops._chunk_scan_states_fwd(Cd, pd, dAd, seq_idx=sd)
+    assert yb.dtype == C.dtype
+    _check("scan_states.lowp", yb.float(), want, 1e-2, 1e-2)
+    # accumulate: added to what the output holds, on a strided view of a wider buffer
+    wide = torch.randn(want.shape[0], want.shape[1], want.shape[2], want.shape[3] + 8, generator=torch.Generator().manual_seed(1))
+    view = _dev(wide)[..., 8:]
+    got = ops._chunk_scan_states_fwd(Cd, pd, dAd, seq_idx=sd, out=view, accumulate=True)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == view.data_ptr()
+    _check("scan_states.accumulate", view, want + wide[..., 8:])
+
+
+def test_chunk_scan_states_cfg2_row(ops, oracle):
+    # one batch row of the Mamba2-2.7B layer shape at full sequence length, states produced by the fused kernel
+    d = oracle.make_inputs(2, b=1)
+    dA = d["dA_cumsum"]
+    xd, Bd, dtd, dAd, Cd = map(_dev, (d["x"], d["B"], d["dt"], dA, d["C"]))
+    prev, _ = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32, initial_states=_dev(d["initial_states"]))
+    y = ops._chunk_scan_states_fwd(Cd, prev, dAd, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = oracle.chunk_scan_states_ref(d["C"], prev.cpu(), dA)
+    _check("scan_states.cfg2row", y, want)
+    # size-independent property: linear in C -- exact for a power of two, up to terms at the denormal threshold
+    # (states of fast-decaying heads are that small, and the matrix cores flush what falls below it)
+    y2 = ops._chunk_scan_states_fwd(Cd * 2.0, prev, dAd, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    err = float((y2 - y * 2.0).abs().max())
+    print(f"[scan_states.linearity] max_abs={err:.3e}", flush=True)
+    assert err <= 1e-30
+
+
 # ------------------------------------------------------------------ the path inside a whole SSD forward
 @pytest.mark.parametrize("kw", [dict(), dict(nseq=4, L=900, init=True)], ids=["plain", "varlen-ragged-init"])
 def test_whole_ssd_forward_with_library_kernels(ops, oracle, kw):

@@ -408,3 +408,37 @@ def test_chunk_scan_special_cases(oracle):
         for m in range(Q):
             want = sum(cb[0, c, 0, m, k] * x[0, c * Q + k] for k in range(m + 1)) + x[0, c * Q + m] * D[:, None]
             assert torch.allclose(y[0, c * Q + m], want, atol=1e-5)
+
+
+def test_chunk_scan_states_is_the_state_half_of_the_chunk_scan(oracle):
+    o = oracle
+    # (1) with cb = 0 (no intra-chunk term, no D) the pinned chunk scan reduces to its state half: ragged last chunk,
+    #     grouped C, packed sequences
+    d = o.make_inputs(0, b=2, L=200, H=4, G=2, P=8, N=16, Q=64, nseq=3)
+    g = torch.Generator().manual_seed(3)
+    states = torch.randn(2, 4, 4, 8, 16, generator=g)
+    cb0 = torch.zeros(2, 4, 2, 64, 64)
+    for seq in (None, d["seq_idx"]):
+        want, _ = o.chunk_scan_ref(cb0, d["x"], d["dt"], d["dA_cumsum"], d["C"], states, seq_idx=seq)
+        got = o.chunk_scan_states_ref(d["C"], states, d["dA_cumsum"], seq_idx=seq)
+        assert got.shape == want.shape and torch.allclose(got, want, rtol=1e-6, atol=1e-6)
+    # (2) brute force on a tiny case, element by element, with the first chunk's sequence ids != 0 (scale 0 there:
+    #     the previous id of chunk 0 is taken as 0) and a change of sequence inside chunk 1
+    b, L, H, P, N, Q = 1, 6, 2, 2, 3, 4
+    C = torch.randn(b, L, 1, N, generator=g)
+    st = torch.randn(b, 2, H, P, N, generator=g)
+    dA = -torch.rand(b, H, 2, Q, generator=g)
+    seq = torch.tensor([[1, 1, 1, 1, 1, 2]], dtype=torch.int32)
+    got = o.chunk_scan_states_ref(C, st, dA, seq_idx=seq)
+    for l in range(L):
+        c, m = divmod(l, Q)
+        prev = int(seq[0, c * Q - 1]) if c else 0
+        for h in range(H):
+            for p in range(P):
+                dot = sum(float(C[0, l, 0, n]) * float(st[0, c, h, p, n]) for n in range(N))
+                want = dot * math.exp(float(dA[0, h, c, m])) if int(seq[0, l]) == prev else 0.0
+                assert abs(float(got[0, l, h, p]) - want) < 1e-5, (l, h, p)
+    assert float(got[0, :4].abs().max()) == 0.0 and float(got[0, 4].abs().max()) > 0 and float(got[0, 5].abs().max()) == 0.0
+    # (3) linear in the states and in C
+    got2 = o.chunk_scan_states_ref(2 * C, st * -0.5, dA, seq_idx=seq)
+    assert torch.allclose(got2, -got, atol=1e-6)
