@@ -118,8 +118,20 @@ def main():
     def cumsum(i):
         return ssd_amd._chunk_cumsum_fwd(raw[i % nsets], A_dev, cfg["Q"], dt_bias=bias_dev, dt_softplus=True)
 
+    # the consumer of the passed states (state half of the chunk scan), fp32 y, on the states of the timed launches
+    C_dev = [mv(d["C"]).clone() for _ in range(nsets)]
+    prev_states = [fused(i)[0] for i in range(nsets)]
+    y_bufs = [torch.empty(b, L, H, P, device=dev) for _ in range(nsets)]
+
+    def scan_states(i):
+        s = sets[i % nsets]
+        return ssd_amd._chunk_scan_states_fwd(C_dev[i % nsets], prev_states[i % nsets], s["dA_cumsum"], seq_idx=s["seq_idx"],
+                                              out=y_bufs[i % nsets])
+
     _, bf16_ev = timed(fused_bf16, max(5, args.steps // 4), 3)
     _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
+    _, scan_ev = timed(scan_states, max(5, args.steps // 4), 3)
+    del prev_states, y_bufs
 
     # parity of what was timed, on one batch row, against the CPU oracle
     out, fin = fused(0)
@@ -161,6 +173,7 @@ def main():
         "unfused_us": round(unf_ev * 1e6, 2),
         "fused_bf16_out_us": round(bf16_ev * 1e6, 2),
         "chunk_cumsum_us": round(cs_ev * 1e6, 2),
+        "chunk_scan_states_us": round(scan_ev * 1e6, 2),
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,
     }

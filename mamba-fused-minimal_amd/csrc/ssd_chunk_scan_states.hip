@@ -63,8 +63,9 @@ template <int NK, int PB> constexpr int state_lds() { return PB * 16 * NK * 32 *
 template <int NK, int PB> constexpr int wave_lds() { return 2 * 16 * NK * 32 * 2 + 16 * PB * 16 * 4; }   // 2 C blocks + y block
 template <int NK, int PB> constexpr int lds_bytes() { return state_lds<NK, PB>() + 4 * wave_lds<NK, PB>(); }
 
-// NK = dstate / 32 (2 or 4); PB = headdim rows of the item / 16 (2 or 4); MB = 16-token blocks per wave = Q / 64.
-template <int NK, int PB, int MB>
+// NK = dstate / 32 (2 or 4); PB = headdim rows of the item / 16 (2 or 4); MB = 16-token blocks per wave = Q / 64;
+// PLAIN = y is fp32 and overwritten (the element-type and accumulate branches fold away).
+template <int NK, int PB, int MB, bool PLAIN>
 __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 {
     constexpr int N = 32 * NK;
@@ -218,15 +219,21 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 #pragma unroll
         for (int j = 0; j < PB; ++j)
             *(f32x4 *)(obuf + i16 * (OP * 16) + ((((4 * j + kg) ^ i16) & (OP - 1)) << 4)) = acc[j] * sc[mb];
+        f32x4 yv[PB];
+#pragma unroll
+        for (int r = 0; r < PB; ++r) {
+            const int t = r * (64 / OP) + lane / OP;
+            yv[r] = *(const f32x4 *)(obuf + t * (OP * 16) + ((((lane % OP) ^ t) & (OP - 1)) << 4));
+        }
 #pragma unroll
         for (int r = 0; r < PB; ++r) {
             const int t = r * (64 / OP) + lane / OP;
             const int piece = lane % OP;
-            f32x4 v = *(const f32x4 *)(obuf + t * (OP * 16) + (((piece ^ t) & (OP - 1)) << 4));
+            f32x4 v = yv[r];
             const int voff = t * (int)o_pitch + 4 * piece;              // elements, from the block's first token
             const int soff = (tok0 + 16 * mb) * (int)o_pitch;
-            if (p.dt_out == DT_F32) {
-                if (p.accumulate) {
+            if (PLAIN || p.dt_out == DT_F32) {
+                if (!PLAIN && p.accumulate) {
                     const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(rsO, 4 * voff, 4 * soff, 0);
                     v += __builtin_bit_cast(f32x4, o);
                 }
@@ -311,29 +318,30 @@ bool scan_states_mfma_supported(const ScanParams &p)
     return (int64_t)p.batch * p.C * p.nheads * (p.headdim / 32) < 0x7fffffffLL;
 }
 
-template <int NK, int PB, int MB>
+template <int NK, int PB, int MB, bool PLAIN>
 static hipError_t launch_scan_k(const ScanParams &p, hipStream_t s)
 {
     constexpr int lds = scan::lds_bytes<NK, PB>();
     static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
     if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_kernel<NK, PB, MB>,
+        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_kernel<NK, PB, MB, PLAIN>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         configured = true;
     }
     const int64_t items = (int64_t)p.batch * p.C * p.nheads * (p.headdim / (16 * PB));
-    hipLaunchKernelGGL((scan::scan_states_kernel<NK, PB, MB>), dim3((unsigned)items), dim3(256), lds, s, p);
+    hipLaunchKernelGGL((scan::scan_states_kernel<NK, PB, MB, PLAIN>), dim3((unsigned)items), dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
 template <int NK, int PB>
 static hipError_t launch_scan_q(const ScanParams &p, hipStream_t s)
 {
+    const bool plain = p.dt_out == DT_F32 && !p.accumulate;
     switch (p.Q) {
-    case 64: return launch_scan_k<NK, PB, 1>(p, s);
-    case 128: return launch_scan_k<NK, PB, 2>(p, s);
-    default: return launch_scan_k<NK, PB, 4>(p, s);
+    case 64: return plain ? launch_scan_k<NK, PB, 1, true>(p, s) : launch_scan_k<NK, PB, 1, false>(p, s);
+    case 128: return plain ? launch_scan_k<NK, PB, 2, true>(p, s) : launch_scan_k<NK, PB, 2, false>(p, s);
+    default: return plain ? launch_scan_k<NK, PB, 4, true>(p, s) : launch_scan_k<NK, PB, 4, false>(p, s);
     }
 }
 
