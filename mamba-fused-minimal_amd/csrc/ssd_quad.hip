@@ -143,38 +143,48 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     const int32_t *sqb = HAS_SEQ ? p.seq + b * p.ssq_b : nullptr;
 
     // ---- request helpers -------------------------------------------------------------------------------------
-    // B block `it` of a step = 32 tokens x 16 columns (32 bytes per token), 64 pieces of 16 bytes; lane l deposits
-    // its piece at byte 16*l of the block.  Piece l = (column half l/32, token bit 2 = (l/16)%2, position l%16) with
-    // token = position%4 + 4*((l/16)%2) + 8*(position/4): the 16 tokens that one transposing read touches then
-    // lie at the 16 different positions, i.e. on different LDS banks.
-    const int Blane = (int)(((lane & 3) | (((lane >> 4) & 1) << 2) | (((lane >> 2) & 3) << 3)) * Brb) + 16 * (lane >> 5);
-    auto load_B = [&](__amdgpu_buffer_rsrc_t rs, int s, int it) {       // step s of the chunk behind rs
+    // A step's B tile (32 tokens x dstate) sits in LDS as NT blocks of 1 KB, block (th, pair) = 16 tokens (token
+    // half th) x 32 columns (column pair `pair`), row-major: one request fetches a block, lane l the 16 bytes
+    // (token l/4, piece l%4) -- four adjacent lanes read 64 contiguous bytes, which the memory pipeline merges into
+    // one request (every lane in another row would cost four times the cycles there) -- and deposits them at byte
+    // 16*l.  For the tokens 8..15 of a block the two 32-byte halves are swapped (piece ^ 2), see the reads below.
+    const int Blane = (int)((lane >> 2) * Brb) + 16 * ((lane & 3) ^ ((lane >> 5) << 1));
+    auto load_B = [&](__amdgpu_buffer_rsrc_t rs, int s, int bi) {       // block bi of step s of the chunk behind rs
 #if defined(__HIP_DEVICE_COMPILE__)      // the LDS address space does not exist in the host pass
         typedef __attribute__((address_space(3))) void *lds_ptr;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRing) * NT + it) * 1024), 16, Blane,
-                                                 (int)(32 * s * Brb) + 32 * it, 0, 0);
+        const int th = bi / (NT / 2), pair = bi % (NT / 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRing) * NT + bi) * 1024), 16, Blane,
+                                                 (int)((32 * s + 16 * th) * Brb) + 64 * pair, 0, 0);
 #else
-        (void)rs; (void)s; (void)it; (void)Blane;
+        (void)rs; (void)s; (void)bi; (void)Blane;
 #endif
     };
-    // The transposing read for (block it, tokens 8kg + 4*half .. +3): lane (i16, kg) addresses the 8 bytes of
-    // token 8kg + 4*half + i16/4, columns 4*(i16%4)..+3 and receives column i16 of those four tokens.
+    // The transposing read for (16 columns `it`, tokens 8kg + 4*half .. +3): lane (i16, kg) addresses the 8 bytes
+    // of token 8kg + 4*half + i16/4, columns 4*(i16%4)..+3 of that column block and receives column i16 of those
+    // four tokens.  Token 8kg + 4*half + j is row 8*(kg%2) + 4*half + j of block (kg/2, it/2), and the column block
+    // is the 32-byte half it%2 of the row -- swapped for kg odd, so that the lane groups kg and kg + 1, 512 bytes
+    // apart, touch different banks.  Btr[it%2] holds the lane's part of the address.
     // The reads are written as inline assembly with explicit s_waitcnt: given the intrinsic, the compiler orders
     // every such read behind ALL outstanding loads that write LDS (s_waitcnt vmcnt(0)), which would serialise the
     // three-steps-ahead requests with their use.
-    uint32_t Btr = (((i16 & 3) >> 1) * 2) * 256 + ((i16 >> 2) | (kg << 2)) * 16 + (i16 & 1) * 8;   // + 256 * half
+    uint32_t Btr[2];
+    Btr[0] = (kg >> 1) * (NT / 2) * 1024 + (8 * (kg & 1) + (i16 >> 2)) * 64 + (kg & 1) * 32 + (i16 & 3) * 8;   // + 256 * half
+    Btr[1] = Btr[0] ^ 32;
 #if defined(__HIP_DEVICE_COMPILE__)
-    Btr += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
+    Btr[0] += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
+    Btr[1] += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
 #endif
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Wunused-lambda-capture"   // the host pass sees no use of Btr
-    auto read_Bt = [&, Btr](auto offc, u32x2 &lo, u32x2 &hi) {        // offc: byte offset of the block in the ring
-        constexpr int off = decltype(offc)::value;
+    const uint32_t Btr0 = Btr[0], Btr1 = Btr[1];
+    auto read_Bt = [&, Btr0, Btr1](auto slotc, auto itc, u32x2 &lo, u32x2 &hi) {    // ring slot, column block
+        constexpr int it = decltype(itc)::value;
+        constexpr int off = (decltype(slotc)::value * NT + (it >> 1)) * 1024;
 #if defined(__HIP_DEVICE_COMPILE__)
         asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
-                     : "=&v"(lo), "=&v"(hi) : "v"(Btr), "n"(off), "n"(off + 256) : "memory");
+                     : "=&v"(lo), "=&v"(hi) : "v"((it & 1) ? Btr1 : Btr0), "n"(off), "n"(off + 256) : "memory");
 #else
-        lo = hi = (u32x2){0u, 0u}; (void)Btr; (void)off;
+        lo = hi = (u32x2){0u, 0u}; (void)Btr0; (void)Btr1; (void)off;
 #endif
     };
 #pragma clang diagnostic pop
@@ -259,7 +269,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         const uint32_t r0 = xr[2 * q], r1_ = xr[2 * q + 1];
         const float v0 = __builtin_bit_cast(float, jp ? (r0 & 0xffff0000u) : (r0 << 16)) * wv[2 * q];
         const float v1 = __builtin_bit_cast(float, jp ? (r1_ & 0xffff0000u) : (r1_ << 16)) * wv[2 * q + 1];
-        const uint32_t hp = pack_bf16(v0, v1);
+        uint32_t hp = pack_bf16(v0, v1);
+        asm volatile("" : "+v"(hp));      // keeps the compiler from converting v0 a second time to get h0
         const float h0 = __builtin_bit_cast(float, hp << 16);
         const float h1 = __builtin_bit_cast(float, hp & 0xffff0000u);
         f.hi[jp][q] = hp;
@@ -357,7 +368,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         __builtin_amdgcn_sched_barrier(0);
         static_for<kAhead>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            read_Bt(std::integral_constant<int, i * 1024>{}, blo[i], bhi[i]);
+            read_Bt(std::integral_constant<int, 0>{}, ic, blo[i], bhi[i]);
         });
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -421,8 +432,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
             }
             {
                 constexpr int tn = it + kAhead;     // block kAhead iterations on: this step's tile or the next one's
-                constexpr int blk = tn < NT ? (s % kRing) * NT + tn : ((s + 1) % kRing) * NT + tn - NT;
-                read_Bt(std::integral_constant<int, blk * 1024>{}, blo[tn % 4], bhi[tn % 4]);
+                read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
+                        blo[tn % 4], bhi[tn % 4]);
             }
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
