@@ -145,6 +145,14 @@ int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states
                               void *stream);
 
 /*
+ * Tuning / test hook with no counterpart in the reference: which matrix-core kernel serves ssd_chunk_scan_states_fwd
+ * where both apply.  0 = let the library choose (the default); 1 = one workgroup per (batch, chunk, head);
+ * 2 = one workgroup per run of heads, with the chunk's C rows kept in LDS across the run (needs headdim % 64 == 0
+ * and contiguous dA_cumsum rows; other calls are served as with 0).  Returns the previous setting, or SSD_ERR_SHAPE.
+ */
+int ssd_set_scan_kernel(int kernel);
+
+/*
  * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
  * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
  * waves per state tile; 1 = one wave per state tile (the fused kernel with four tiles per workgroup) wherever that

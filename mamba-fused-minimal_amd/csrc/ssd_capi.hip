@@ -261,6 +261,12 @@ int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states
     return (int)ssd::launch_scan_states(p, (hipStream_t)stream);
 }
 
+int ssd_set_scan_kernel(int kernel)
+{
+    if (kernel < 0 || kernel > 2) return SSD_ERR_SHAPE;
+    return ssd::set_scan_kernel(kernel);
+}
+
 int ssd_set_token_split(int waves)
 {
     if (waves != 0 && waves != 1 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;

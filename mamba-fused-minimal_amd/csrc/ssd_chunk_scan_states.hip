@@ -59,6 +59,43 @@ __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t rs, char *dst
 #endif
 }
 
+// Four consecutive values of one y row (element offsets voff per lane + soff uniform) in y's element type,
+// optionally added to what is there.  PLAIN: fp32, overwrite.  The data registers of a wide store are read out over
+// several cycles after issue; the wait states that depend on them keep a following writer of the same registers away.
+template <bool PLAIN>
+__device__ __forceinline__ void store_y(__amdgpu_buffer_rsrc_t rsO, int dt_out, int accumulate, int voff, int soff, f32x4 v)
+{
+    if (PLAIN || dt_out == DT_F32) {
+        if (!PLAIN && accumulate) {
+            const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(rsO, 4 * voff, 4 * soff, 0);
+            v += __builtin_bit_cast(f32x4, o);
+        }
+        const u32x4 q = __builtin_bit_cast(u32x4, v);
+        __builtin_amdgcn_raw_buffer_store_b128(q, rsO, 4 * voff, 4 * soff, 0);
+        asm volatile("s_nop 3" ::"v"(q) : "memory");
+    } else {
+        const bool bf = dt_out == DT_BF16;
+        if (accumulate) {
+            const u32x2 o = __builtin_amdgcn_raw_buffer_load_b64(rsO, 2 * voff, 2 * soff, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t w = (e & 1) ? (o[e >> 1] >> 16) : (o[e >> 1] & 0xffffu);
+                v[e] += bf ? bf16_bits_to_f32(w) : (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+            }
+        }
+        u32x2 q;
+        if (bf) {
+            q = (u32x2){pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+        } else {
+            typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+            const h2 a = {(_Float16)v.x, (_Float16)v.y}, d = {(_Float16)v.z, (_Float16)v.w};
+            q = (u32x2){__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, d)};
+        }
+        __builtin_amdgcn_raw_buffer_store_b64(q, rsO, 2 * voff, 2 * soff, 0);
+        asm volatile("s_nop 3" ::"v"(q) : "memory");
+    }
+}
+
 template <int NK, int PB> constexpr int state_lds() { return PB * 16 * NK * 32 * 4; }          // rows x dstate fp32
 template <int NK, int PB> constexpr int wave_lds() { return 2 * 16 * NK * 32 * 2 + 16 * PB * 16 * 4; }   // 2 C blocks + y block
 template <int NK, int PB> constexpr int lds_bytes() { return state_lds<NK, PB>() + 4 * wave_lds<NK, PB>(); }
@@ -232,36 +269,171 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
             f32x4 v = yv[r];
             const int voff = t * (int)o_pitch + 4 * piece;              // elements, from the block's first token
             const int soff = (tok0 + 16 * mb) * (int)o_pitch;
-            if (PLAIN || p.dt_out == DT_F32) {
-                if (!PLAIN && p.accumulate) {
-                    const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(rsO, 4 * voff, 4 * soff, 0);
-                    v += __builtin_bit_cast(f32x4, o);
-                }
-                const u32x4 q = __builtin_bit_cast(u32x4, v);
-                __builtin_amdgcn_raw_buffer_store_b128(q, rsO, 4 * voff, 4 * soff, 0);
-                asm volatile("s_nop 3" ::"v"(q) : "memory");
-            } else {
-                const bool bf = p.dt_out == DT_BF16;
-                if (p.accumulate) {
-                    const u32x2 o = __builtin_amdgcn_raw_buffer_load_b64(rsO, 2 * voff, 2 * soff, 0);
+            store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, soff, v);
+        }
+    }
+}
+
+// Second decomposition, for headdim % 64 == 0 and contiguous dA_cumsum rows: one workgroup takes one (batch, chunk),
+// a block of 64 headdim rows and a run of `hb` heads of one group.  The chunk's C rows are fetched once into LDS
+// and serve every head of the run; the state block of head i + 1 is requested (into the other half of a double
+// buffer) before the work on head i starts, so its latency hides behind 128 MFMAs per wave.  Wave w owns the 16
+// rows p0 + 16w .. + 15 of the block for ALL tokens of the chunk: the state is converted to bf16 hi + lo once per
+// head and wave (not once per wave as above would need for whole rows), and a wave's results are 64 contiguous bytes
+// per token, passed through 1 KB of LDS so that four adjacent lanes write them.
+template <int NK, int MBT> constexpr int heads_lds()       // C tile + 2 state blocks + 2 dA_cumsum rows + 4 y blocks
+{
+    return 16 * MBT * NK * 64 + 2 * 64 * NK * 128 + 2 * 1024 + 4 * 1024;     // chunk_size <= 256: a row fits 1 KB
+}
+
+// NK = dstate / 32; MBT = chunk_size / 16
+template <int NK, int MBT, bool PLAIN>
+__global__ void __launch_bounds__(256, 1) scan_states_heads_kernel(const ScanParams p, int hb)
+{
+    constexpr int N = 32 * NK, Q = 16 * MBT;
+    constexpr int PRS = N / 4, PRC = N / 8;
+    constexpr int SI = 64 * PRS / 64 / 4;        // state load instructions per wave and head
+    constexpr int CI = Q * PRC / 64 / 4;         // C load instructions per wave
+    static_assert(Q * 4 <= 1024, "one request fetches a dA_cumsum row");
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    char *cld = lds;                                      // [Q tokens][N bf16], pieces swizzled
+    char *sld = cld + Q * N * 2;                          // 2 x [64 rows][N fp32], pieces swizzled
+    char *dld = sld + 2 * 64 * N * 4;                     // 2 x 1 KB: [Q] fp32 (a request always deposits 1 KB)
+    char *obuf = dld + 2 * 1024 + wave * 1024;            // [16 tokens][64 bytes], pieces swizzled
+
+    const int n_pt = p.headdim >> 6;
+    const int runs = p.nheads / hb;
+    int item = blockIdx.x;
+    const int pt = item % n_pt; item /= n_pt;
+    const int run = item % runs; item /= runs;
+    const int c = item % p.C;
+    const int b = item / p.C;
+    const int h0 = run * hb;
+    const int g = h0 / (p.nheads / p.ngroups);
+    const int p0 = pt * 64;
+
+    // tokens of this chunk whose sequence differs from the one the chunk's incoming state belongs to: bit mb of
+    // `dead` = token 16 mb + i16 (kernels/ssd_chunk_scan.py:86-88, 101-104)
+    uint32_t dead = 0;
+    if (p.seq) {
+        const int32_t prev = c >= 1 ? p.seq[b * p.ssq_b + (int64_t)(c * Q - 1) * p.ssq_l] : 0;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t w = (e & 1) ? (o[e >> 1] >> 16) : (o[e >> 1] & 0xffffu);
-                        v[e] += bf ? bf16_bits_to_f32(w) : (float)__builtin_bit_cast(_Float16, (uint16_t)w);
-                    }
-                }
-                u32x2 q;
-                if (bf) {
-                    q = (u32x2){pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
-                } else {
-                    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
-                    const h2 a = {(_Float16)v.x, (_Float16)v.y}, d = {(_Float16)v.z, (_Float16)v.w};
-                    q = (u32x2){__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, d)};
-                }
-                __builtin_amdgcn_raw_buffer_store_b64(q, rsO, 2 * voff, 2 * soff, 0);
-                asm volatile("s_nop 3" ::"v"(q) : "memory");
+        for (int mb = 0; mb < MBT; ++mb) {
+            const int l = c * Q + 16 * mb + i16;
+            const int32_t id = l < p.seqlen ? p.seq[b * p.ssq_b + (int64_t)l * p.ssq_l] : -1;
+            dead |= (id != prev ? 1u : 0u) << mb;
+        }
+    }
+
+    // ---- requests.  State block and dA_cumsum row of head i -> buffer i % 2.
+    const int64_t s_pitch = p.sst_p * 4;
+    auto request_head = [&](int i) {
+        const int h = h0 + i;
+        const auto rsS = make_rsrc((const char *)p.states + 4 * (b * p.sst_b + c * p.sst_c + h * p.sst_h + (int64_t)p0 * p.sst_p),
+                                   (int64_t)63 * s_pitch + N * 4);
+#pragma unroll
+        for (int k = 0; k < SI; ++k) {
+            const int ins = wave * SI + k;
+            const int row = ins * (64 / PRS) + lane / PRS;
+            const int q = (lane % PRS) ^ (row & 15);
+            load_to_lds(rsS, sld + (i & 1) * 64 * N * 4 + ins * 1024, row * (int)s_pitch + q * 16, 0);
+        }
+        if (wave == 0) {
+            const auto rsD = make_rsrc(p.dacs + b * p.sda_b + h * p.sda_h + c * p.sda_c, Q * 4);
+            load_to_lds(rsD, dld + (i & 1) * 1024, 16 * lane, 0);      // lanes past the row are out of range: zeros
+        }
+    };
+    {
+        const int64_t c_pitch = p.sC_l * 2;
+        const auto rsC = make_rsrc((const char *)p.Cm + 2 * (b * p.sC_b + g * p.sC_g), (int64_t)(p.seqlen - 1) * c_pitch + N * 2);
+#pragma unroll
+        for (int k = 0; k < CI; ++k) {
+            const int ins = wave * CI + k;
+            const int t = ins * (64 / PRC) + lane / PRC;                // token within the chunk
+            const int q = (lane % PRC) ^ (t & (PRC - 1));
+            load_to_lds(rsC, cld + ins * 1024, t * (int)c_pitch + q * 16, c * Q * (int)c_pitch);
+        }
+    }
+    request_head(0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int64_t o_pitch = p.so_l;
+    const int esz = p.dt_out == DT_F32 ? 4 : 2;
+    const int voff = (lane >> 2) * (int)o_pitch + 4 * (lane & 3);       // after the pass through LDS: token lane / 4
+    char *owr = obuf + i16 * 64 + ((kg ^ (i16 >> 2)) << 4);
+    const char *ord = obuf + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4);
+
+    for (int i = 0; i < hb; ++i) {
+        // Everything requested for head i (and, the first time, the C tile) has landed: behind those requests this
+        // wave only issued the stores of head i - 1.  The compiler does not track loads that write LDS, so the wait
+        // is explicit; the barrier publishes the other waves' parts and tells that every wave is done with head
+        // i - 1, whose buffers the requests for head i + 1 overwrite.
+        if (i == 0) __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(MBT));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (i + 1 < hb) request_head(i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+
+        const int h = h0 + i;
+        // this wave's 16 state rows as A operands: hi + lo bf16 of row 16 wave + i16, dstate 32 ks + 8 kg .. + 7
+        u32x4 shi[NK], slo[NK];
+        const char *rowp = sld + (i & 1) * 64 * N * 4 + (16 * wave + i16) * (N * 4);
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) {
+            const int q0 = 8 * ks + 2 * kg;
+            const f32x4 a = *(const f32x4 *)(rowp + ((q0 ^ i16) << 4));
+            const f32x4 d = *(const f32x4 *)(rowp + (((q0 + 1) ^ i16) << 4));
+            const float v[8] = {a.x, a.y, a.z, a.w, d.x, d.y, d.z, d.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t hp = pack_bf16(v[2 * e], v[2 * e + 1]);
+                asm volatile("" : "+v"(hp));
+                const float f0 = __builtin_bit_cast(float, hp << 16);
+                const float f1 = __builtin_bit_cast(float, hp & 0xffff0000u);
+                shi[ks][e] = hp;
+                slo[ks][e] = pack_bf16(v[2 * e] - f0, v[2 * e + 1] - f1);
             }
         }
+        const auto rsO = make_rsrc((char *)p.out + esz * (b * p.so_b + h * p.so_h + p0 + 16 * wave),
+                                   ((int64_t)(p.seqlen - 1) * o_pitch + 16) * esz);
+        const float *dal = (const float *)(dld + (i & 1) * 1024);
+
+        // Software pipeline over the 16-token blocks: the C operands of block mb + 1 are read before the MFMAs of
+        // block mb, and a block's result is written to LDS, read back (issued at once: LDS operations of a wave
+        // execute in order) and stored only after the MFMAs of the next block, so that no LDS latency is waited for.
+        auto read_C = [&](int mb, bf16x8 (&cf)[NK]) {
+            const char *cb = cld + (16 * mb + i16) * (PRC * 16);
+#pragma unroll
+            for (int ks = 0; ks < NK; ++ks)
+                cf[ks] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(cb + ((((4 * ks + kg) ^ i16) & (PRC - 1)) << 4)));
+        };
+        bf16x8 cfn[NK];
+        read_C(0, cfn);
+        f32x4 vprev = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mb = 0; mb < MBT; ++mb) {
+            bf16x8 cf[NK];
+#pragma unroll
+            for (int ks = 0; ks < NK; ++ks) cf[ks] = cfn[ks];
+            if (mb + 1 < MBT) read_C(mb + 1, cfn);
+            float sc = __expf(dal[16 * mb + i16]);
+            if ((dead >> mb) & 1) sc = 0.f;
+            // two independent accumulation chains (hi and lo halves of the state)
+            f32x4 ah = {0.f, 0.f, 0.f, 0.f}, al = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NK; ++ks) {
+                ah = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[ks]), cf[ks], ah, 0, 0, 0);
+                al = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[ks]), cf[ks], al, 0, 0, 0);
+            }
+            if (mb > 0) store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (c * Q + 16 * (mb - 1)) * (int)o_pitch, vprev);
+            // acc[r] = y[token 16 mb + i16][row 4 kg + r]: through LDS to (token lane / 4, 16-byte piece lane % 4)
+            *(f32x4 *)owr = (ah + al) * sc;
+            vprev = *(const f32x4 *)ord;
+        }
+        store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (c * Q + 16 * (MBT - 1)) * (int)o_pitch, vprev);
     }
 }
 
@@ -345,9 +517,67 @@ static hipError_t launch_scan_q(const ScanParams &p, hipStream_t s)
     }
 }
 
+template <int NK, int MBT, bool PLAIN>
+static hipError_t launch_heads_k(const ScanParams &p, int hb, hipStream_t s)
+{
+    constexpr int lds = scan::heads_lds<NK, MBT>();
+    static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
+    if (lds > 65536 && !configured) {
+        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_heads_kernel<NK, MBT, PLAIN>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const int64_t items = (int64_t)p.batch * p.C * (p.nheads / hb) * (p.headdim / 64);
+    hipLaunchKernelGGL((scan::scan_states_heads_kernel<NK, MBT, PLAIN>), dim3((unsigned)items), dim3(256), lds, s, p, hb);
+    return hipGetLastError();
+}
+
+template <int NK, int MBT>
+static hipError_t launch_heads_q(const ScanParams &p, int hb, hipStream_t s)
+{
+    return p.dt_out == DT_F32 && !p.accumulate ? launch_heads_k<NK, MBT, true>(p, hb, s) : launch_heads_k<NK, MBT, false>(p, hb, s);
+}
+
+static int g_scan_kernel = 0;       // 0 = choose, 1 = one workgroup per head, 2 = runs of heads
+
+int set_scan_kernel(int k)
+{
+    const int old = g_scan_kernel;
+    g_scan_kernel = k;
+    return old;
+}
+
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s)
 {
     if ((int64_t)p.batch * p.seqlen * p.nheads * p.headdim == 0) return hipSuccess;
+    if (scan_states_mfma_supported(p) && g_scan_kernel != 1 && p.headdim % 64 == 0 && p.sda_k == 1 &&
+        ((uintptr_t)p.dacs % 16) == 0 && (p.sda_b | p.sda_h | p.sda_c) % 4 == 0) {
+        // runs of heads: the longest divisor of the heads per group up to 10 (enough workgroups to fill the chip
+        // matter more than the last bit of C reuse)
+        const int per_group = p.nheads / p.ngroups;
+        int hb = 1;
+        for (int d = 2; d <= 10; ++d)
+            if (per_group % d == 0) hb = d;
+        const bool small = (int64_t)p.batch * p.C * (p.nheads / hb) * (p.headdim / 64) < 512;
+        // measured at the Mamba2-2.7B layer shape: 229 us against 257 us for fp32 y written plainly; with bf16 y or
+        // accumulation the one-workgroup-per-head kernel is the faster one (196 / 419 us against 208 / 576 us)
+        const bool plain = p.dt_out == DT_F32 && !p.accumulate;
+        if (g_scan_kernel == 2 || (!small && plain)) {
+            if (p.dstate == 128) {
+                switch (p.Q) {
+                case 64: return launch_heads_q<4, 4>(p, hb, s);
+                case 128: return launch_heads_q<4, 8>(p, hb, s);
+                default: return launch_heads_q<4, 16>(p, hb, s);
+                }
+            }
+            switch (p.Q) {
+            case 64: return launch_heads_q<2, 4>(p, hb, s);
+            case 128: return launch_heads_q<2, 8>(p, hb, s);
+            default: return launch_heads_q<2, 16>(p, hb, s);
+            }
+        }
+    }
     if (scan_states_mfma_supported(p)) {
         const bool wide = p.headdim % 64 == 0;
         if (p.dstate == 128) return wide ? launch_scan_q<4, 4>(p, s) : launch_scan_q<4, 2>(p, s);

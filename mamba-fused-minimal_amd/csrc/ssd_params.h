@@ -117,6 +117,7 @@ hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);
 bool scan_states_mfma_supported(const ScanParams &p);
+int set_scan_kernel(int k);       // 0 = automatic; 1 = one workgroup per head; 2 = runs of heads; returns the old value
 int set_token_split(int wv);      // 0 = automatic; 2 or 4 forces the token split of the MFMA kernels; returns the old value
 
 }  // namespace ssd

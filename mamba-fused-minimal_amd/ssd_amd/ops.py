@@ -216,6 +216,15 @@ def _chunk_scan_states_fwd(C, prev_states, dA_cumsum, seq_idx=None, out=None, ou
     return out
 
 
+def set_scan_kernel(kernel):
+    """Tuning / test hook (no counterpart in the reference): 1 = the scan consumer runs one workgroup per head, 2 = one
+    workgroup per run of heads wherever that kernel applies, 0 = let the library choose.  Returns the previous setting."""
+    rc = _lib.load().ssd_set_scan_kernel(int(kernel))
+    if rc < 0:
+        raise ValueError("scan kernel must be 0, 1 or 2")
+    return rc
+
+
 def set_token_split(waves):
     """Tuning / test hook (no counterpart in the reference): 2 or 4 = the token-split bf16 MFMA kernels with that
     many waves per state tile, 1 = the fused kernel with one wave per tile and four tiles per workgroup wherever it

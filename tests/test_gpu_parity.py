@@ -310,9 +310,20 @@ def test_chunk_cumsum_strided_dt_and_pipeline(ops, oracle):
     dict(L=300, H=3, P=40, N=24, G=1, Q=64),             # nothing aligned: plain FMA kernel
     dict(dtype="fp16"),                                  # fp16 C: plain FMA kernel
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
-def test_chunk_scan_states(ops, oracle, kw):
+@pytest.mark.parametrize("kernel", [1, 2])
+def test_chunk_scan_states(ops, oracle, kw, kernel):
+    # kernel: both matrix-core decompositions in turn (the library picks by problem size; shapes that the forced
+    # one does not take fall through to the other or to the plain kernel)
     base = dict(b=2, L=1024, H=6, G=1, init=True)
     base.update(kw)
+    old = ops.set_scan_kernel(kernel)
+    try:
+        _scan_states_case(ops, oracle, base)
+    finally:
+        ops.set_scan_kernel(old)
+
+
+def _scan_states_case(ops, oracle, base):
     d = oracle.make_inputs(1, **base)
     C, seq, dA = d["C"], d["seq_idx"], d["dA_cumsum"]
     prev, _ = oracle.fused_ref(d["B"], d["x"], d["dt"], dA, initial_states=d["initial_states"], seq_idx=seq)
