@@ -129,6 +129,22 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
                          int dt_softplus, float dt_min, float dt_max, void *stream);
 
 /*
+ * dt preparation + chunk state + state passing in one call: ssd_chunk_cumsum_fwd followed by
+ * ssd_fused_chunk_state_passing_fwd (reference: kernels/ssd_chunk_state.py:176-199 followed by
+ * kernels/fused_globalbar.py:201-266 / kernels/fused_concurrent.py:255-331, as main.py:78-100 calls them).
+ * dt_raw: (batch, seqlen, nheads) f32/bf16/f16; A, dt_bias (nullable): (nheads).  dt_out and dA_cumsum
+ * (batch, nheads, nchunks, chunk_size) fp32 are OUTPUTS here (the stages after the path read them); the other
+ * arguments are those of ssd_fused_chunk_state_passing_fwd without `states`.  Two launches on `stream`; dt_out and
+ * dA_cumsum are exactly what ssd_chunk_cumsum_fwd writes.
+ */
+int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
+                                             const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *seq_idx,
+                                             const ssd_tensor *initial_states, const ssd_tensor *dt_out,
+                                             const ssd_tensor *dA_cumsum, const ssd_tensor *out,
+                                             const ssd_tensor *final_states, const ssd_dims *dims, int dt_softplus,
+                                             float dt_min, float dt_max, int clamp, void *stream);
+
+/*
  * The consumer of the passed states: the state-dependent half of the chunk scan.  Replaces that part of
  * _chunk_scan_fwd_kernel (kernels/ssd_chunk_scan.py:94-117; wrapper _chunk_scan_fwd, :172-224):
  *   y[b,cQ+m,h,p] = scale_m * sum_n C[b,cQ+m,h/(H/G),n] * prev_states[b,c,h,p,n],

@@ -123,14 +123,12 @@ int ssd_chunk_state_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tens
     return run(p, false, stream);
 }
 
-int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
-                                      const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
-                                      const ssd_tensor *initial_states, const ssd_tensor *states,
-                                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims,
-                                      int clamp, void *stream)
+// Fills Params for a fused call (chunk state + state passing).
+static int fill_fused(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                      const ssd_tensor *seq_idx, const ssd_tensor *initial_states, const ssd_tensor *states,
+                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, int clamp)
 {
     if (!present(out) || !present(final_states)) return SSD_ERR_NULL;
-    Params p;
     int rc = fill_common(p, x, B, dt, dA_cumsum, seq_idx, states, dims, clamp);
     if (rc) return rc;
     if (!dtype_ok(out->dtype) || final_states->dtype != SSD_F32) return SSD_ERR_DTYPE;
@@ -145,6 +143,42 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
         p.init = initial_states->data; p.dt_init = initial_states->dtype;
         p.sin_b = initial_states->stride[0]; p.sin_h = initial_states->stride[1]; p.sin_p = initial_states->stride[2];
     }
+    return SSD_OK;
+}
+
+int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                      const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                      const ssd_tensor *initial_states, const ssd_tensor *states,
+                                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims,
+                                      int clamp, void *stream)
+{
+    Params p;
+    int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, states, out, final_states, dims, clamp);
+    if (rc) return rc;
+    return run(p, true, stream);
+}
+
+int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
+                                             const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *seq_idx,
+                                             const ssd_tensor *initial_states, const ssd_tensor *dt_out,
+                                             const ssd_tensor *dA_cumsum, const ssd_tensor *out,
+                                             const ssd_tensor *final_states, const ssd_dims *dims, int dt_softplus,
+                                             float dt_min, float dt_max, int clamp, void *stream)
+{
+    if (!present(dt_raw) || !present(A)) return SSD_ERR_NULL;
+    if (!dtype_ok(dt_raw->dtype) || !dtype_ok(A->dtype)) return SSD_ERR_DTYPE;
+    if (present(dt_bias) && !dtype_ok(dt_bias->dtype)) return SSD_ERR_DTYPE;
+    Params p;
+    int rc = fill_fused(p, x, B, dt_out, dA_cumsum, seq_idx, initial_states, nullptr, out, final_states, dims, clamp);
+    if (rc) return rc;
+    // Two launches on the caller's stream.  A variant of the fused kernel that computes dt / dA_cumsum per chunk
+    // itself was built and measured: each of its workgroups walks two heads through the whole sequence and has to
+    // gather their two columns out of the token-major dt rows (a request per token and wave), which cost more
+    // (270 against 240 microseconds for both stages at batch 4 x 8192 tokens x 80 heads) than the producer's
+    // transposing pass and the read-back of its 21 MB.
+    rc = ssd_chunk_cumsum_fwd(dt_raw, A, dt_bias, dt_out, dA_cumsum, dims->batch, dims->seqlen, dims->nheads, dims->chunk_size,
+                              dt_softplus, dt_min, dt_max, stream);
+    if (rc) return rc;
     return run(p, true, stream);
 }
 

@@ -8,8 +8,8 @@
 // HBM-bound streaming work with a transpose in the middle: dt arrives token-major (heads contiguous), the outputs
 // are head-major (the chunk's tokens contiguous).  A workgroup takes one (batch, chunk) and a tile of 32 heads:
 // reads are 32 consecutive heads per token, the tile is transposed through LDS, and each wave then owns whole head
-// rows: a lane holds EPL consecutive tokens, sums them serially, the 64 lane totals are scanned with DPP-free
-// shuffles, and both outputs leave as contiguous rows.
+// rows: a lane holds EPL consecutive tokens, sums them serially, the 64 lane totals are scanned with
+// data-parallel-primitive moves, and both outputs leave as contiguous rows.
 #include "ssd_params.h"
 
 namespace ssd {
@@ -92,12 +92,7 @@ __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
             tot[i] = run[i];
         }
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1)
-#pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                const float o = __shfl_up(tot[i], d, 64);
-                if (lane >= d) tot[i] += o;
-            }
+        for (int i = 0; i < NR; ++i) tot[i] = wave_inclusive_sum(tot[i]);
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             const int r = r0 + 4 * i, hr = h0 + r;

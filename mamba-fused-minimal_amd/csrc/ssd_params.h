@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <utility>
 
 namespace ssd {
 
@@ -104,6 +105,26 @@ __device__ __forceinline__ void store_from_f32(void *base, int64_t idx, int dt, 
     if (dt == DT_F32) ((float *)base)[idx] = v;
     else if (dt == DT_BF16) ((uint16_t *)base)[idx] = f32_to_bf16_bits(v);
     else ((_Float16 *)base)[idx] = (_Float16)v;
+}
+
+// Inclusive sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS traffic): shifts by 1, 2, 4, 8
+// inside each row of 16 lanes, then lane 15 of a row added to the whole next row, then lane 31 to the upper half.
+__device__ __forceinline__ float wave_inclusive_sum(float x)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    auto shifted = [](float v, auto ctrl, auto rows) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value,
+                                                                     decltype(rows)::value, 0xf, true));
+    };
+    using std::integral_constant;
+    x += shifted(x, integral_constant<int, 0x111>{}, integral_constant<int, 0xf>{});     // row_shr:1
+    x += shifted(x, integral_constant<int, 0x112>{}, integral_constant<int, 0xf>{});     // row_shr:2
+    x += shifted(x, integral_constant<int, 0x114>{}, integral_constant<int, 0xf>{});     // row_shr:4
+    x += shifted(x, integral_constant<int, 0x118>{}, integral_constant<int, 0xf>{});     // row_shr:8
+    x += shifted(x, integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{});     // row_bcast:15 into rows 1, 3
+    x += shifted(x, integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{});     // row_bcast:31 into rows 2, 3
+#endif
+    return x;
 }
 
 // Launchers implemented in the .hip files; each returns the hipError_t of its launch.

@@ -175,6 +175,49 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
     return dA_cumsum, dt_out
 
 
+def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dtype, dt_bias=None, dt_softplus=False,
+                                                dt_limit=(0.0, float("inf")), initial_states=None, seq_idx=None,
+                                                _clamp=True):
+    """``_chunk_cumsum_fwd`` followed by ``_fused_chunk_state_state_passing_fwd`` in one call (the first three stages of
+    the reference's main.py:78-100): dt is the raw (batch, seqlen, nheads) tensor.  Returns
+    (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32, dA_cumsum, dt_out (b,H,C,Q) fp32)."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, seqlen, nheads)
+    assert A.shape == (nheads,)
+    if dt_bias is not None:
+        assert dt_bias.shape == (nheads,)
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+        if seq_idx.dtype != torch.int32:
+            seq_idx = seq_idx.to(torch.int32)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+        if initial_states.stride(-1) != 1:
+            initial_states = initial_states.contiguous()
+    _lib.require_device(x, "_fused_cumsum_chunk_state_state_passing_fwd")
+    nchunks = math.ceil(seqlen / chunk_size)
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if B.stride(-1) != 1:
+        B = B.contiguous()
+    dt_out = torch.empty(batch, nheads, nchunks, chunk_size, device=x.device, dtype=torch.float32)
+    dA_cumsum = torch.empty(batch, nheads, nchunks, chunk_size, device=x.device, dtype=torch.float32)
+    out = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=out_dtype or torch.float32)
+    final_states = torch.empty((batch, nheads, headdim, dstate), device=x.device, dtype=torch.float32)
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    T = _lib.tensor_arg
+    with torch.cuda.device(x.device):
+        rc = _lib.load().ssd_fused_cumsum_chunk_state_passing_fwd(
+            T(x), T(B), T(dt), T(A), T(dt_bias), T(seq_idx), T(initial_states), T(dt_out), T(dA_cumsum), T(out),
+            T(final_states), dims, int(bool(dt_softplus)), float(dt_limit[0]), float(dt_limit[1]), 1 if _clamp else 0,
+            _stream(x))
+    _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd")
+    return out, final_states, dA_cumsum, dt_out
+
+
 def _chunk_scan_states_fwd(C, prev_states, dA_cumsum, seq_idx=None, out=None, out_dtype=None, accumulate=False):
     """The state-consuming half of the reference's ``_chunk_scan_fwd`` (kernels/ssd_chunk_scan.py:94-117, wrapper
     :172-224): y[b,cQ+m,h,:] = scale_m * (C[b,cQ+m,g,:] . prev_states[b,c,h]), scale_m = exp(dA_cumsum[b,h,c,m]) where

@@ -299,6 +299,42 @@ def test_chunk_cumsum_strided_dt_and_pipeline(ops, oracle):
     _check("pipeline.final", fin, want_fin)
 
 
+# ------------------------------------------------------------------ dt preparation + fused path in one call
+@pytest.mark.parametrize("kw", [
+    dict(),                                              # chunk 256, dstate 128
+    dict(L=1000, nseq=5),                                # ragged last chunk + packed sequences
+    dict(Q=128, L=1024, N=64, H=8, G=2),                 # chunk 128, dstate 64, grouped B
+    dict(dtype="fp32", L=512),                           # fp32 inputs
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
+def test_fused_with_dt_preparation(ops, oracle, kw):
+    # one call for cumsum -> fused: against the same composition of the oracle, and the dt / dA_cumsum it returns
+    # against the library's stand-alone producer bit for bit
+    base = dict(b=2, L=1024, H=6, G=1, init=True)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    Q = d["cfg"]["Q"]
+    raw, A, bias, seq, init = d["dt_raw"], d["A"], d["dt_bias"], d["seq_idx"], d["initial_states"]
+    for softplus, use_bias, limit in ((True, True, (0.0, float("inf"))), (False, False, (1e-3, 0.1))):
+        b_ = bias if use_bias else None
+        want_da, want_dt = oracle.chunk_cumsum_ref(raw, A, Q, dt_bias=b_, dt_softplus=softplus, dt_limit=limit)
+        want_out, want_fin = oracle.fused_ref(d["B"], d["x"], want_dt, want_da, initial_states=init, seq_idx=seq)
+        out, fin, dA, dt = ops._fused_cumsum_chunk_state_state_passing_fwd(
+            _dev(d["B"]), _dev(d["x"]), _dev(raw), _dev(A), Q, torch.float32, dt_bias=_dev(b_), dt_softplus=softplus,
+            dt_limit=limit, initial_states=_dev(init), seq_idx=_dev(seq))
+        torch.cuda.synchronize()
+        tag = f"prep+fused[{softplus}]"
+        _check(tag + ".dt", dt, want_dt, 2e-6, 1e-9)
+        _check(tag + ".dA_cumsum", dA, want_da, 1e-5, 1e-6)
+        _check(tag + ".out", out, want_out)
+        _check(tag + ".final", fin, want_fin)
+        dA2, dt2 = ops._chunk_cumsum_fwd(_dev(raw), _dev(A), Q, dt_bias=_dev(b_), dt_softplus=softplus, dt_limit=limit)
+        out2, fin2 = ops._fused_chunk_state_state_passing_fwd(_dev(d["B"]), _dev(d["x"]), dt2, dA2, torch.float32,
+                                                              initial_states=_dev(init), seq_idx=_dev(seq))
+        torch.cuda.synchronize()
+        assert torch.equal(dt2, dt) and torch.equal(dA2, dA), tag
+        assert torch.equal(out2, out) and torch.equal(fin2, fin), tag
+
+
 # ------------------------------------------------------------------ the consumer of the passed states
 @pytest.mark.parametrize("kw", [
     dict(),                                              # chunk 256, dstate 128, headdim 64: matrix-core kernel
