@@ -152,6 +152,9 @@ def test_config4_long_grouped_slicewise(ops, oracle):
     dict(L=300, H=3, P=40, N=24, G=1, Q=64),             # nothing aligned: generic path
     dict(dtype="fp16"),                                  # fp16 inputs: generic path
     dict(b=3, L=256, H=5),                               # a single chunk
+    dict(L=1),                                           # a single token
+    dict(L=33, nseq=2),                                  # one ragged chunk holding two sequences
+    dict(L=257, H=8),                                    # one full chunk and one token (four-tile kernel when forced)
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
 def test_small_variants(ops, oracle, kw):
     base = dict(b=2, L=1024, H=6, G=1, init=True)
@@ -166,6 +169,8 @@ def test_small_variants(ops, oracle, kw):
     dict(Q=128, L=1024),                                 # chunk 128
     dict(N=64),                                          # dstate 64
     dict(P=128, H=4, G=2),                               # headdim 128, grouped B
+    dict(L=1),                                           # a single token
+    dict(L=257),                                         # one full chunk and one token
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
 def test_token_split_variants(ops, oracle, kw, waves):
     # every bf16 MFMA kernel family (the library picks one from the problem size by itself): one wave per tile
