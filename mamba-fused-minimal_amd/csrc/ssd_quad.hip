@@ -92,8 +92,9 @@ struct Frag { uint32_t hi[2][4], lo[2][4]; };
 constexpr int kRingSteps = 4;
 template <int SPC> constexpr int ring_of() { return kRingSteps <= SPC ? kRingSteps : 4; }
 
-template <int NT, int SPC> constexpr int wave_lds() { return ring_of<SPC>() * 2048 + 3 * 32 * SPC * 4; }     // x ring + weights
-constexpr int kStage = 1024;        // per wave: one 16 x 16 fp32 block of the state on its way to memory
+// x ring + two weight slots: a chunk's weights are written half a chunk ahead, while the current chunk's are in use
+template <int NT, int SPC> constexpr int wave_lds() { return ring_of<SPC>() * 2048 + 2 * 32 * SPC * 4; }
+constexpr int kStage = 2048;        // per wave: two 16 x 16 fp32 blocks of the state on their way to memory
 template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * NT * 1024 + 4 * (wave_lds<NT, SPC>() + kStage); }
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (chunk_size / 32: 4 or 8);
@@ -110,7 +111,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     char *bring = lds;                                                   // kRing x NT blocks of 1 KB, shared
     char *xring = lds + kRing * NT * 1024 + wave * wave_lds<NT, SPC>();  // kRing slots x (32 tokens x 64 bytes)
-    char *wbuf = xring + kRing * 2048;                                   // 3 slots x Q weights
+    char *wbuf = xring + kRing * 2048;                                   // 2 slots x Q weights
     char *stage = lds + kRing * NT * 1024 + 4 * wave_lds<NT, SPC>() + wave * kStage;
 
     // Work item -> (batch, head, row slice); the four items of a workgroup share batch and group (checked on the
@@ -292,6 +293,46 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         const int voff = (p0 + 2 * (lane >> 2)) * row_pitch + 4 * (lane & 3);
         f32x4 *wr = (f32x4 *)(stage + i16 * 64 + ((kg ^ (i16 >> 2)) << 4));
         const f32x4 *rd = (const f32x4 *)(stage + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4));
+        if (dt != DT_F32) {
+            // 16-bit destination: the two blocks (it, jp = 0 / 1) -- the same 16 columns of adjacent rows -- go
+            // through LDS together and come back as (lane/4 = row pair, (lane/2)%2 = jp, lane%2 = 8 columns), so
+            // that every lane stores 16 bytes: half the store instructions of the 32-bit case
+            const int i = lane >> 2, jq = (lane >> 1) & 1, half = lane & 1;
+            const int voff2 = (p0 + 2 * i + jq) * row_pitch + 8 * half;
+            const char *rd2 = stage + jq * 1024 + i * 64;
+            char *wr1 = stage + 1024 + i16 * 64 + ((kg ^ (i16 >> 2) ^ 1) << 4);
+            const int sw = (i >> 2) ^ jq;       // block 1 is shifted by one column group: the two blocks of a read
+                                                // instruction then sit on different banks
+            // (the pair it + 1 is written and read back -- LDS operations of a wave execute in order -- before the
+            // pair it is converted and stored, so that its reads have returned by then)
+            f32x4 a[NT], d[NT];
+#pragma unroll
+            for (int k = 0; k <= NT; ++k) {
+                if (k < NT) {
+                    *wr = acc[k][0];
+                    *(f32x4 *)((char *)wr1) = acc[k][1];
+                    a[k] = *(const f32x4 *)(rd2 + (((2 * half) ^ sw) << 4));
+                    d[k] = *(const f32x4 *)(rd2 + (((2 * half + 1) ^ sw) << 4));
+                }
+                if (k >= 1) {
+                    const int it = k - 1;
+                    const f32x4 u = a[it], w = d[it];
+                    u32x4 q;
+                    if (dt == DT_BF16) {
+                        q = (u32x4){pack_bf16(u.x, u.y), pack_bf16(u.z, u.w), pack_bf16(w.x, w.y), pack_bf16(w.z, w.w)};
+                    } else {
+                        typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+                        const h2 e0 = {(_Float16)u.x, (_Float16)u.y}, e1 = {(_Float16)u.z, (_Float16)u.w};
+                        const h2 e2 = {(_Float16)w.x, (_Float16)w.y}, e3 = {(_Float16)w.z, (_Float16)w.w};
+                        q = (u32x4){__builtin_bit_cast(uint32_t, e0), __builtin_bit_cast(uint32_t, e1),
+                                    __builtin_bit_cast(uint32_t, e2), __builtin_bit_cast(uint32_t, e3)};
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b128(q, rs, 2 * voff2, 2 * (16 * it), 0);
+                    asm volatile("s_nop 3" ::"v"(q) : "memory");
+                }
+            }
+            return;
+        }
         // LDS operations of one wave execute in order, so block k + 1 may be written right behind the read of
         // block k; the store of a block follows kLag blocks later, when its read has long returned
         constexpr int kLag = 4;
@@ -354,7 +395,9 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     // four MFMAs of one iteration, so a single block in flight would leave the matrix pipe waiting every iteration.
     constexpr int kAhead = 3;
     static_assert(NT % 4 == 0 && kAhead < 4 && kAhead <= NT, "slot of a block = its tile index % 4");
-    constexpr int kStores = 2 * NT;     // vector-memory operations of one store_state
+    // vector-memory operations of one store_state, at least (a 16-bit `out` takes NT stores, a 32-bit one 2 NT; the
+    // waits below may count fewer operations than were issued, never more)
+    constexpr int kStores = F32IO ? 2 * NT : NT;
     u32x2 blo[4], bhi[4];
     {
         // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
@@ -389,7 +432,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
         if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
-        else read_operands(0, (ws + 1) % 3, xr, wv);
+        else read_operands(0, ws ^ 1, xr, wv);
 
         if (s == 0) {
             // chunk boundary: out[:, c] = state entering the chunk, then s <- exp(dA_chunk) * s
@@ -447,11 +490,11 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
             if (s == 1 && it == NT - 1) mnext = load_meta(c + 1);
             __builtin_amdgcn_sched_barrier(0);
         });
-        if (s == SPC / 2) put_weights(c + 1, (ws + 1) % 3, mnext);
+        if (s == SPC / 2) put_weights(c + 1, ws ^ 1, mnext);
     };
 
     for (int c = 0; c < C; ++c) {
-        const int ws = c % 3;
+        const int ws = c & 1;
         step(c, std::integral_constant<int, 0>{}, ws, fA, fB);
         step(c, std::integral_constant<int, 1>{}, ws, fB, fA);
         step(c, std::integral_constant<int, 2>{}, ws, fA, fB);
