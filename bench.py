@@ -21,7 +21,7 @@ HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
 # HBM bytes per fused launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB -> bytes; the
 # factors are what the same counters read for a plain 1 GiB copy).  Keyed by workload name; see the rocprof summaries
 # kept with the repository.  None = not measured for that workload / kernel version.
-MEASURED_TRAFFIC_BYTES = {"cfg2_mamba2_2p7b": 730515098}
+MEASURED_TRAFFIC_BYTES = {"cfg2_mamba2_2p7b": 730515354}
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 
 
