@@ -171,12 +171,21 @@ int ssd_set_scan_kernel(int kernel);
 /*
  * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
  * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
- * waves per state tile; 1 = one wave per state tile (the fused kernel with four tiles per workgroup) wherever that
+ * waves per state tile; 1 = one wave per state tile (the kernel with four tiles per workgroup) wherever that
  * kernel applies.  The setting holds for every later call of this process.  Returns the previous setting, or
  * SSD_ERR_SHAPE for any other value.  Results agree between the settings to rounding (the tokens are summed in
  * another order), not bit for bit.
  */
 int ssd_set_token_split(int waves);
+
+/*
+ * Tuning / test hook with no counterpart in the reference: how many consecutive chunks a workgroup of the
+ * four-tiles-per-workgroup kernel walks when that kernel serves ssd_chunk_state_fwd (chunk states are independent of
+ * each other, so a sequence is cut into segments that run as separate workgroups).  0 = let the library choose from
+ * the problem size (the default); values above the number of chunks mean one segment.  The results do not depend on
+ * the setting, bit for bit.  Returns the previous setting, or SSD_ERR_SHAPE for a negative value.
+ */
+int ssd_set_segment_chunks(int chunks);
 
 #ifdef __cplusplus
 }

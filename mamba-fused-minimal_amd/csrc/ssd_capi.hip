@@ -86,6 +86,9 @@ int run(const Params &p, bool fused, void *stream)
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
     if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
+    else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 2048)) &&
+             ssd::quad_chunk_state_supported(p))
+        e = ssd::launch_quad_chunk_state(p, s);
     else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
     return (int)e;
 }
@@ -299,6 +302,12 @@ int ssd_set_scan_kernel(int kernel)
 {
     if (kernel < 0 || kernel > 2) return SSD_ERR_SHAPE;
     return ssd::set_scan_kernel(kernel);
+}
+
+int ssd_set_segment_chunks(int chunks)
+{
+    if (chunks < 0) return SSD_ERR_SHAPE;
+    return ssd::set_quad_segment_chunks(chunks);
 }
 
 int ssd_set_token_split(int waves)

@@ -33,6 +33,7 @@ struct Params {
     int dt_in, dt_states, dt_out, dt_init;
     int clamp;
     int n_items;          // work items of the launch
+    int n_seg;            // segments the chunks are split into (chunk-state launch of the four-tile kernel)
 };
 
 // State passing on a flattened state axis.
@@ -134,6 +135,9 @@ hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
 hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state tiles per workgroup sharing B in LDS
 bool quad_supported(const Params &p);
+hipError_t launch_quad_chunk_state(const Params &p, hipStream_t s);     // chunk states only, same kernel
+bool quad_chunk_state_supported(const Params &p);
+int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup of the above; returns the old value
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

@@ -99,7 +99,10 @@ template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * N
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (chunk_size / 32: 4 or 8);
 // F32IO = out and initial states are fp32 (or the latter absent): element-type branches fold away.
-template <int NT, int SPC, bool HAS_SEQ, bool F32IO>
+// CO = chunk states only (kernels/ssd_chunk_state.py:202-232): a workgroup walks p.n_seg-th of the chunks, the
+// accumulators restart from zero at every chunk boundary and what they held goes to states[:, c - 1]; nothing is
+// carried from chunk to chunk, so the segments of a sequence are independent workgroups.
+template <int NT, int SPC, bool HAS_SEQ, bool F32IO, bool CO>
 __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
 {
     constexpr int Q = 32 * SPC;
@@ -117,19 +120,30 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     // Work item -> (batch, head, row slice); the four items of a workgroup share batch and group (checked on the
     // host).  Consecutive workgroups sit on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so a
     // batch's B is fetched from HBM by one or two L2 slices only.
-    const int per_xcd = ((p.n_items >> 2) + 7) >> 3;                     // workgroups per XCD
-    const int wg = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if (4 * wg >= p.n_items) return;                                     // whole workgroup: no barrier is skipped
+    const int n_wg = p.n_items >> 2, n_seg = CO ? p.n_seg : 1;
+    const int per_xcd = (n_wg * n_seg + 7) >> 3;                         // workgroups per XCD
+    const int vwg = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (vwg >= n_wg * n_seg) return;                                     // whole workgroup: no barrier is skipped
+    int wg = vwg, c0 = 0, c1 = p.C;
+    if (CO) {
+        // (batch, segment) pairs one after the other: the workgroups running side by side on an XCD read the
+        // same B rows
+        const int wpb = n_wg / p.batch, bs = vwg / wpb, cps = (p.C + n_seg - 1) / n_seg;
+        wg = (bs / n_seg) * wpb + vwg % wpb;
+        c0 = (bs % n_seg) * cps;
+        c1 = min(p.C, c0 + cps);
+        if (c0 >= c1) return;
+    }
     const int item = 4 * wg + wave;
     const int n_pt = p.headdim >> 5;
     const int pt = item % n_pt;
     const int r1 = item / n_pt;
     const int h = r1 % p.nheads;
     const int b = r1 / p.nheads;
-    const int C = p.C, L = p.seqlen;
+    const int C = c1, L = p.seqlen;      // chunks at and beyond c1 are not this workgroup's: never requested
     const int g = h / (p.nheads / p.ngroups);
     const int p0 = pt * 32;
-    const int dt_out = F32IO ? (int)DT_F32 : p.dt_out, dt_init = F32IO ? (int)DT_F32 : p.dt_init;
+    const int dt_out = F32IO ? (int)DT_F32 : (CO ? p.dt_states : p.dt_out), dt_init = F32IO ? (int)DT_F32 : p.dt_init;
 
     const char *xrow = (const char *)p.x + 2 * (b * p.sx_b + h * p.sx_h);
     const char *Brow = (const char *)p.B + 2 * (b * p.sB_b + g * p.sB_g);
@@ -268,20 +282,22 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     // tokens (2q, 2q+1) of headdim row 2*i16 + jp: x * w in fp32, split into bf16 hi + bf16 lo
     auto frag_piece = [&](int q, int jp, const uint32_t (&xr)[8], const float (&wv)[8], Frag &f) {
         const uint32_t r0 = xr[2 * q], r1_ = xr[2 * q + 1];
-        const float v0 = __builtin_bit_cast(float, jp ? (r0 & 0xffff0000u) : (r0 << 16)) * wv[2 * q];
-        const float v1 = __builtin_bit_cast(float, jp ? (r1_ & 0xffff0000u) : (r1_ << 16)) * wv[2 * q + 1];
-        uint32_t hp = pack_bf16(v0, v1);
-        asm volatile("" : "+v"(hp));      // keeps the compiler from converting v0 a second time to get h0
+        const float x0 = __builtin_bit_cast(float, jp ? (r0 & 0xffff0000u) : (r0 << 16));
+        const float x1 = __builtin_bit_cast(float, jp ? (r1_ & 0xffff0000u) : (r1_ << 16));
+        uint32_t hp = pack_bf16(x0 * wv[2 * q], x1 * wv[2 * q + 1]);
+        asm volatile("" : "+v"(hp));      // keeps the compiler from converting the product a second time to get h0
         const float h0 = __builtin_bit_cast(float, hp << 16);
         const float h1 = __builtin_bit_cast(float, hp & 0xffff0000u);
         f.hi[jp][q] = hp;
-        f.lo[jp][q] = pack_bf16(v0 - h0, v1 - h1);
+        // the residual of the exact product, as a fused multiply-add everywhere: left to the compiler, some copies
+        // of this code would subtract from the rounded product instead and the bits would depend on the copy
+        f.lo[jp][q] = pack_bf16(__builtin_fmaf(x0, wv[2 * q], -h0), __builtin_fmaf(x1, wv[2 * q + 1], -h1));
     };
 
     // ---- state ---------------------------------------------------------------------------------------------
     // acc[it][jp][r]: dstate column 16*it + 4*kg + r of headdim row p0 + 2*i16 + jp
     f32x4 acc[NT][2];
-    const int64_t slice_out = (int64_t)(p.headdim - 1) * p.so_p + p.dstate;
+    const int64_t slice_out = (int64_t)(p.headdim - 1) * (CO ? p.sst_p : p.so_p) + p.dstate;
     const int64_t slice_fin = (int64_t)(p.headdim - 1) * p.sf_p + p.dstate;
     auto store_state = [&](__amdgpu_buffer_rsrc_t rs, int dt, int row_pitch) {
         // The accumulators hold a 16 x 16 block as (lane%16 = row, lane/16 = group of four columns): neighbouring
@@ -354,7 +370,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp) {
             acc[it][jp] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            if (p.init) {
+            if (!CO && p.init) {
                 const int64_t off = b * p.sin_b + h * p.sin_h + (int64_t)(p0 + 2 * i16 + jp) * p.sin_p + 16 * it + 4 * kg;
                 if (dt_init == DT_F32) {
                     acc[it][jp] = *(const f32x4 *)((const float *)p.init + off);
@@ -377,9 +393,9 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         *(u32x4 *)(bring + (i * 4 + wave) * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
     __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): the zeros are in place before any row lands
     __builtin_amdgcn_s_barrier();
-    Meta mcur = load_meta(0);
-    __amdgpu_buffer_rsrc_t rsx0 = chunk_rsrc(xrow, xrb, 0), rsx1 = chunk_rsrc(xrow, xrb, 1);
-    __amdgpu_buffer_rsrc_t rsB0 = chunk_rsrc(Brow, Brb, 0), rsB1 = chunk_rsrc(Brow, Brb, 1);
+    Meta mcur = load_meta(c0);
+    __amdgpu_buffer_rsrc_t rsx0 = chunk_rsrc(xrow, xrb, c0), rsx1 = chunk_rsrc(xrow, xrb, c0 + 1);
+    __amdgpu_buffer_rsrc_t rsB0 = chunk_rsrc(Brow, Brb, c0), rsB1 = chunk_rsrc(Brow, Brb, c0 + 1);
     // requests of the steps 0..kDist-1, in the order (x, x, B...) that every later step keeps
 #pragma unroll
     for (int s = 0; s < kDist; ++s) {
@@ -388,7 +404,7 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         for (int k = 0; k < NTW; ++k) load_B(rsB0, s, wave * NTW + k);
         __builtin_amdgcn_sched_barrier(0);
     }
-    put_weights(0, 0, mcur);
+    put_weights(c0, 0, mcur);
     Frag fA, fB;
     // B operands (transposed blocks) travel kAhead iterations ahead of the MFMAs that use them, across step
     // boundaries: block t of the stream of (step, tile) pairs sits in slot t % 4.  An LDS read takes longer than the
@@ -434,7 +450,19 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
         else read_operands(0, ws ^ 1, xr, wv);
 
-        if (s == 0) {
+        if (CO && s == 0) {
+            // chunk boundary: states[:, c - 1] = what the previous chunk summed up, then start again from zero.  The
+            // first chunk of the segment has nothing to hand over: its stores go through a descriptor of extent
+            // zero, which drops them -- the waits count a boundary's stores whether or not they reach memory.
+            const int cp = c > c0 ? c - 1 : c0;
+            store_state(make_rsrc((char *)p.states + (b * p.sst_b + cp * p.sst_c + h * p.sst_h) * esize_of(dt_out),
+                                  c > c0 ? slice_out * esize_of(dt_out) : 0), dt_out, (int)p.sst_p);
+#pragma unroll
+            for (int it = 0; it < NT; ++it)
+#pragma unroll
+                for (int jp = 0; jp < 2; ++jp) acc[it][jp] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+        if (!CO && s == 0) {
             // chunk boundary: out[:, c] = state entering the chunk, then s <- exp(dA_chunk) * s
             store_state(make_rsrc((char *)p.out + (b * p.so_b + c * p.so_c + h * p.so_h) * esize_of(dt_out),
                                   slice_out * esize_of(dt_out)), dt_out, (int)p.so_p);
@@ -493,8 +521,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         if (s == SPC / 2) put_weights(c + 1, ws ^ 1, mnext);
     };
 
-    for (int c = 0; c < C; ++c) {
-        const int ws = c & 1;
+    for (int c = c0; c < C; ++c) {
+        const int ws = (c - c0) & 1;
         step(c, std::integral_constant<int, 0>{}, ws, fA, fB);
         step(c, std::integral_constant<int, 1>{}, ws, fB, fA);
         step(c, std::integral_constant<int, 2>{}, ws, fA, fB);
@@ -510,19 +538,18 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         rsx1 = chunk_rsrc(xrow, xrb, c + 2);
         rsB1 = chunk_rsrc(Brow, Brb, c + 2);
     }
-    store_state(make_rsrc(p.fin + b * p.sf_b + h * p.sf_h, slice_fin * 4), DT_F32, (int)p.sf_p);
+    if (CO)
+        store_state(make_rsrc((char *)p.states + (b * p.sst_b + (C - 1) * p.sst_c + h * p.sst_h) * esize_of(dt_out),
+                              slice_out * esize_of(dt_out)), dt_out, (int)p.sst_p);
+    else
+        store_state(make_rsrc(p.fin + b * p.sf_b + h * p.sf_h, slice_fin * 4), DT_F32, (int)p.sf_p);
 }
 
 static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
 
-}  // namespace quad
-
-// The four-tiles-per-workgroup kernel serves the fused call without a `states` output, for bf16 x / B with 16-byte
-// aligned rows, unit-stride dt / dA_cumsum rows, and head counts that put four tiles of one group in a workgroup.
-bool quad_supported(const Params &p)
+// what both uses of the kernel ask of the inputs
+static bool inputs_ok(const Params &p)
 {
-    using quad::aligned;
-    if (p.states || !p.out || !p.fin) return false;
     if (p.dt_in != DT_BF16) return false;
     if (p.headdim % 32 != 0) return false;
     if (p.dstate != 64 && p.dstate != 128) return false;
@@ -534,35 +561,71 @@ bool quad_supported(const Params &p)
     if (p.sdt_k != 1 || p.sda_k != 1) return false;
     if (!aligned(p.dt, 16) || (p.sdt_b | p.sdt_h | p.sdt_c) % 4) return false;
     if (!aligned(p.dacs, 16) || (p.sda_b | p.sda_h | p.sda_c) % 4) return false;
-    if (!aligned(p.out, 16) || (p.so_b | p.so_c | p.so_h | p.so_p) % 4) return false;
-    if (!aligned(p.fin, 16) || (p.sf_b | p.sf_h | p.sf_p) % 4) return false;
-    if (p.init && (!aligned(p.init, 16) || (p.sin_b | p.sin_h | p.sin_p) % 4)) return false;
-    if ((int64_t)p.headdim * p.so_p >= (1LL << 28) || (int64_t)p.headdim * p.sf_p >= (1LL << 28)) return false;
     return true;
 }
 
-template <int NT, int SPC, bool SEQ, bool F32IO>
+// rows of 16-byte pieces: fp32 rows start on multiples of 4 elements, 16-bit rows on multiples of 8
+static bool rows_ok(const void *ptr, int dt, int64_t strides_or, int64_t row_stride, int headdim)
+{
+    return aligned(ptr, 16) && strides_or % (dt == DT_F32 ? 4 : 8) == 0 && (int64_t)headdim * row_stride < (1LL << 28);
+}
+
+}  // namespace quad
+
+// The four-tiles-per-workgroup kernel serves the fused call without a `states` output, for bf16 x / B with 16-byte
+// aligned rows, unit-stride dt / dA_cumsum rows, and head counts that put four tiles of one group in a workgroup.
+bool quad_supported(const Params &p)
+{
+    using namespace quad;
+    if (p.states || !p.out || !p.fin) return false;
+    if (!inputs_ok(p)) return false;
+    if (!rows_ok(p.out, p.dt_out, p.so_b | p.so_c | p.so_h | p.so_p, p.so_p, p.headdim)) return false;
+    if (!rows_ok(p.fin, DT_F32, p.sf_b | p.sf_h | p.sf_p, p.sf_p, p.headdim)) return false;
+    if (p.init && !rows_ok(p.init, p.dt_init, p.sin_b | p.sin_h | p.sin_p, p.sin_p, p.headdim)) return false;
+    return true;
+}
+
+// ... and the chunk-state call (`states` only), under the same conditions.
+bool quad_chunk_state_supported(const Params &p)
+{
+    using namespace quad;
+    if (!p.states || p.out || p.fin) return false;
+    if (!inputs_ok(p)) return false;
+    return rows_ok(p.states, p.dt_states, p.sst_b | p.sst_c | p.sst_h | p.sst_p, p.sst_p, p.headdim);
+}
+
+template <int NT, int SPC, bool SEQ, bool F32IO, bool CO>
 static hipError_t launch_quad_k(const Params &p, dim3 grid, hipStream_t s)
 {
     constexpr int lds = quad::lds_bytes<NT, SPC>();
     static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
     if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)quad::quad_kernel<NT, SPC, SEQ, F32IO>,
+        hipError_t e = hipFuncSetAttribute((const void *)quad::quad_kernel<NT, SPC, SEQ, F32IO, CO>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         configured = true;
     }
-    hipLaunchKernelGGL((quad::quad_kernel<NT, SPC, SEQ, F32IO>), grid, dim3(256), lds, s, p);
+    hipLaunchKernelGGL((quad::quad_kernel<NT, SPC, SEQ, F32IO, CO>), grid, dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
-template <int NT, int SPC>
+template <int NT, int SPC, bool CO>
 static hipError_t launch_quad_t(const Params &p, hipStream_t s)
 {
-    dim3 grid((((p.n_items >> 2) + 7) / 8) * 8);
-    const bool f32io = p.dt_out == DT_F32 && (!p.init || p.dt_init == DT_F32);
-    if (p.seq) return f32io ? launch_quad_k<NT, SPC, true, true>(p, grid, s) : launch_quad_k<NT, SPC, true, false>(p, grid, s);
-    return f32io ? launch_quad_k<NT, SPC, false, true>(p, grid, s) : launch_quad_k<NT, SPC, false, false>(p, grid, s);
+    dim3 grid((((p.n_items >> 2) * (CO ? p.n_seg : 1) + 7) / 8) * 8);
+    const bool f32io = CO ? p.dt_states == DT_F32 : p.dt_out == DT_F32 && (!p.init || p.dt_init == DT_F32);
+    if (p.seq) return f32io ? launch_quad_k<NT, SPC, true, true, CO>(p, grid, s) : launch_quad_k<NT, SPC, true, false, CO>(p, grid, s);
+    return f32io ? launch_quad_k<NT, SPC, false, true, CO>(p, grid, s) : launch_quad_k<NT, SPC, false, false, CO>(p, grid, s);
+}
+
+template <bool CO>
+static hipError_t launch_quad_c(const Params &p, hipStream_t s)
+{
+    const int nt = p.dstate / 16, spc = p.Q / 32;
+    if (nt == 8 && spc == 8) return launch_quad_t<8, 8, CO>(p, s);
+    if (nt == 8 && spc == 4) return launch_quad_t<8, 4, CO>(p, s);
+    if (nt == 4 && spc == 8) return launch_quad_t<4, 8, CO>(p, s);
+    return launch_quad_t<4, 4, CO>(p, s);
 }
 
 hipError_t launch_quad(const Params &p_in, hipStream_t s)
@@ -570,11 +633,34 @@ hipError_t launch_quad(const Params &p_in, hipStream_t s)
     Params p = p_in;
     p.n_items = p.batch * p.nheads * (p.headdim / 32);
     if (p.n_items <= 0) return hipSuccess;
-    const int nt = p.dstate / 16, spc = p.Q / 32;
-    if (nt == 8 && spc == 8) return launch_quad_t<8, 8>(p, s);
-    if (nt == 8 && spc == 4) return launch_quad_t<8, 4>(p, s);
-    if (nt == 4 && spc == 8) return launch_quad_t<4, 8>(p, s);
-    return launch_quad_t<4, 4>(p, s);
+    return launch_quad_c<false>(p, s);
+}
+
+static int g_segment_chunks = 0;     // 0 = choose; otherwise the chunks a workgroup walks in the chunk-state launch
+int set_quad_segment_chunks(int n) { const int old = g_segment_chunks; g_segment_chunks = n; return old; }
+
+hipError_t launch_quad_chunk_state(const Params &p_in, hipStream_t s)
+{
+    Params p = p_in;
+    p.n_items = p.batch * p.nheads * (p.headdim / 32);
+    if (p.n_items <= 0 || p.C <= 0) return hipSuccess;
+    // Chunks per workgroup.  Measured times follow  (workgroups per compute unit, rounded up) x (chunks per
+    // workgroup + 0.4): a workgroup's first requests have nothing to hide behind, which costs about 0.4 of a chunk,
+    // and the compute unit with the most workgroups finishes last (b=4 L=8192 H=80: 190 / 162 / 160 / 177 / 219 us
+    // for 1 / 2 / 4 / 8 / 32 chunks per workgroup).
+    int cps = g_segment_chunks;
+    if (cps <= 0) {
+        double best = 0;
+        for (int k = 1; k <= p.C; ++k) {
+            const int nseg = (p.C + k - 1) / k;
+            const int per_cu = ((p.n_items >> 2) * nseg + 255) / 256;
+            const double t = per_cu * (k + 0.4);
+            if (cps <= 0 || t < best) { best = t; cps = k; }
+        }
+    }
+    if (cps > p.C) cps = p.C;
+    p.n_seg = (p.C + cps - 1) / cps;
+    return launch_quad_c<true>(p, s);
 }
 
 }  // namespace ssd

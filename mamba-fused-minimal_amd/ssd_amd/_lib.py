@@ -13,7 +13,7 @@ SSD_F32, SSD_BF16, SSD_F16 = 0, 1, 2
 _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_F16}
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
-           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split")
+           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
 class SsdTensor(ctypes.Structure):
@@ -61,6 +61,8 @@ def load():
     lib.ssd_set_scan_kernel.argtypes = [ctypes.c_int]
     lib.ssd_set_token_split.restype = ctypes.c_int
     lib.ssd_set_token_split.argtypes = [ctypes.c_int]
+    lib.ssd_set_segment_chunks.restype = ctypes.c_int
+    lib.ssd_set_segment_chunks.argtypes = [ctypes.c_int]
     _lib = lib
     return lib
 

@@ -268,9 +268,18 @@ def set_scan_kernel(kernel):
     return rc
 
 
+def set_segment_chunks(chunks):
+    """Tuning / test hook (no counterpart in the reference): consecutive chunks per workgroup when the kernel with
+    four tiles per workgroup serves ``_chunk_state_fwd``; 0 = let the library choose.  Returns the previous setting."""
+    rc = _lib.load().ssd_set_segment_chunks(int(chunks))
+    if rc < 0:
+        raise ValueError("chunks per workgroup must be 0 (automatic) or positive")
+    return rc
+
+
 def set_token_split(waves):
     """Tuning / test hook (no counterpart in the reference): 2 or 4 = the token-split bf16 MFMA kernels with that
-    many waves per state tile, 1 = the fused kernel with one wave per tile and four tiles per workgroup wherever it
+    many waves per state tile, 1 = the kernel with one wave per tile and four tiles per workgroup wherever it
     applies, 0 = let the library choose.  Returns the previous setting."""
     rc = _lib.load().ssd_set_token_split(int(waves))
     if rc < 0:

@@ -186,6 +186,41 @@ def test_token_split_variants(ops, oracle, kw, waves):
         ops.set_token_split(old)
 
 
+@pytest.mark.parametrize("chunks", [0, 1, 3, 64])
+@pytest.mark.parametrize("kw", [
+    dict(L=2304),                                        # 9 chunks: segments of 3 divide them, 1 and 64 do not matter
+    dict(L=2000, nseq=5),                                # ragged last chunk + packed sequences
+    dict(Q=128, L=1408, N=64),                           # 11 chunks of 128, dstate 64
+    dict(P=128, H=4, G=2, L=1280),                       # headdim 128, grouped B, 5 chunks
+    dict(L=1),                                           # a single token
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_chunk_state_segments(ops, oracle, kw, chunks):
+    # _chunk_state_fwd on the kernel with four tiles per workgroup: any cut of the chunks into segments gives the
+    # same bits, for fp32 and 16-bit states, into a strided view as well
+    base = dict(b=2, L=1024, H=6, G=1)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    x, B, dt, dA, seq = map(_dev, (d["x"], d["B"], d["dt"], d["dA_cumsum"], d["seq_idx"]))
+    want = oracle.chunk_state_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], seq_idx=d["seq_idx"])
+    old_split, old_chunks = ops.set_token_split(1), ops.set_segment_chunks(chunks)
+    try:
+        print(f"[segments] x{tuple(x.shape)} chunks/workgroup={chunks}", flush=True)
+        st = ops._chunk_state_fwd(B, x, dt, dA, seq_idx=seq)
+        _check("segments.fp32", st, want)
+        lo = ops._chunk_state_fwd(B, x, dt, dA, seq_idx=seq, states_in_fp32=False)
+        assert lo.dtype == x.dtype
+        _check("segments.bf16", lo, want, 1e-2, 1e-3)
+        b, C, H, P, N = want.shape
+        wide = torch.full((b, C, H, P, 2 * N), float("nan"), device="cuda")
+        ops._chunk_state_fwd(B, x, dt, dA, seq_idx=seq, states=wide[..., N:])
+        assert torch.equal(wide[..., N:], st) and torch.isnan(wide[..., :N]).all()
+        ops.set_segment_chunks(2)
+        assert torch.equal(ops._chunk_state_fwd(B, x, dt, dA, seq_idx=seq), st)
+    finally:
+        ops.set_token_split(old_split)
+        ops.set_segment_chunks(old_chunks)
+
+
 def test_bf16_outputs(ops, oracle):
     d = oracle.make_inputs(1, b=2, L=1024, H=6, init=True)
     _run_case(ops, oracle, d, with_states=False, out_dtype=torch.bfloat16, check_unfused=False, name="bf16out")
