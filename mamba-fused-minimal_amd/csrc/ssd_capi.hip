@@ -74,6 +74,37 @@ int fill_common(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_t
     return SSD_OK;
 }
 
+// The recurrence over `states` as the stand-alone kernel sees it: the (headdim, dstate) plane of a head flattened,
+// dA_chunk = the last column of dA_cumsum.
+PassParams pass_params_of(const Params &p)
+{
+    PassParams q;
+    memset(&q, 0, sizeof(q));
+    q.states = p.states; q.dt_states = p.dt_states;
+    q.sst_b = p.sst_b; q.sst_c = p.sst_c; q.sst_h = p.sst_h;
+    q.da = p.dacs + (int64_t)(p.Q - 1) * p.sda_k;
+    q.sda_b = p.sda_b; q.sda_h = p.sda_h; q.sda_c = p.sda_c;
+    q.init = p.init; q.dt_init = p.dt_init; q.sin_b = p.sin_b; q.sin_h = p.sin_h;
+    q.seq = p.seq; q.ssq_b = p.ssq_b; q.ssq_l = p.ssq_l;
+    q.out = p.out; q.dt_out = p.dt_out; q.so_b = p.so_b; q.so_c = p.so_c; q.so_h = p.so_h;
+    q.fin = p.fin; q.sf_b = p.sf_b; q.sf_h = p.sf_h;
+    q.batch = p.batch; q.C = p.C; q.nheads = p.nheads; q.dim = p.headdim * p.dstate;
+    q.seqlen = p.seqlen; q.Q = p.Q;
+    return q;
+}
+
+// Fused call with `states`: can it run as the chunk-state launch of the four-tile kernel + the recurrence?
+bool pair_supported(const Params &p)
+{
+    if (!p.states || !p.out || !p.fin) return false;
+    if (p.dt_states != ssd::DT_F32) return false;      // the recurrence would start from rounded states
+    // the recurrence walks a head's plane as one row
+    if (p.sst_p != p.dstate || p.so_p != p.dstate || p.sf_p != p.dstate || (p.init && p.sin_p != p.dstate)) return false;
+    Params cs = p;
+    cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
+    return ssd::quad_chunk_state_supported(cs);
+}
+
 int run(const Params &p, bool fused, void *stream)
 {
     int rc = check_device();
@@ -86,6 +117,16 @@ int run(const Params &p, bool fused, void *stream)
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
     if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
+    else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8192)) &&
+             pair_supported(p)) {
+        // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
+        // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
+        // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
+        Params cs = p;
+        cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
+        e = ssd::launch_quad_chunk_state(cs, s);
+        if (e == hipSuccess) e = ssd::launch_state_passing(pass_params_of(p), s);
+    }
     else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 2048)) &&
              ssd::quad_chunk_state_supported(p))
         e = ssd::launch_quad_chunk_state(p, s);
