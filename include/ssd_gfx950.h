@@ -117,6 +117,17 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
 int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
 
 /*
+ * No counterpart in the reference.  1 if ssd_fused_chunk_state_passing_fwd would finish sooner for these arguments
+ * when it is handed a `states` buffer (fp32, (batch, nchunks, nheads, headdim, dstate), contiguous (headdim, dstate)
+ * planes) than without one, 0 if not, negative = rejected.  That is the case for long sequences with few state tiles
+ * (batch * nheads * headdim / 32 below 512): with the buffer the call runs as a chunk-state launch that keeps every
+ * compute unit busy plus a streaming recurrence, without it on a kernel that has one workgroup per tile and walks
+ * the chunks serially.  A caller that does not need the states may pass scratch memory; the library itself never
+ * allocates.  Pure host logic; launches nothing.
+ */
+int ssd_query_fused_wants_states(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
+
+/*
  * dt preparation and per-chunk cumulative sum, the producer of `dt` and `dA_cumsum` for the three calls above.
  * Replaces _chunk_cumsum_fwd / _chunk_cumsum_fwd_kernel (kernels/ssd_chunk_state.py:176-199, 33-79):
  *   d = float(dt[b,l,h]) (+ dt_bias[h]); d = log1p(exp(d)) where dt_softplus and d <= 20; d = clamp(d, dt_min, dt_max);

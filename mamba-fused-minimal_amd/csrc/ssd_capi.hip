@@ -273,6 +273,19 @@ int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dim
     return ssd::mfma_supported(p) ? 1 : 0;
 }
 
+int ssd_query_fused_wants_states(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims)
+{
+    Params p;
+    ssd_tensor f32 = {(void *)16, SSD_F32, 0, {0, 0, 0, 1, 0}};
+    int rc = fill_common(p, x, B, &f32, &f32, nullptr, nullptr, dims, 1);
+    if (rc) return rc;
+    if (g_forced_split == 2 || g_forced_split == 4 || !ssd::quad_inputs_supported(p)) return 0;
+    const int tiles = p.batch * p.nheads * (p.headdim / 32);
+    if (g_forced_split == 1) return 0;                  // the fused four-tile kernel is forced and applies
+    if (tiles >= 512) return 0;                         // ... or chosen
+    return (int64_t)tiles * p.C >= 8192 ? 1 : 0;
+}
+
 int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *dt_out,
                          const ssd_tensor *dA_cumsum, int32_t batch, int32_t seqlen, int32_t nheads, int32_t chunk_size,
                          int dt_softplus, float dt_min, float dt_max, void *stream)

@@ -137,6 +137,7 @@ hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state
 bool quad_supported(const Params &p);
 hipError_t launch_quad_chunk_state(const Params &p, hipStream_t s);     // chunk states only, same kernel
 bool quad_chunk_state_supported(const Params &p);
+bool quad_inputs_supported(const Params &p);     // what the four-tile kernel asks of x, B, dt, dA_cumsum and the shape
 int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup of the above; returns the old value
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);

@@ -585,6 +585,8 @@ bool quad_supported(const Params &p)
     return true;
 }
 
+bool quad_inputs_supported(const Params &p) { return quad::inputs_ok(p); }
+
 // ... and the chunk-state call (`states` only), under the same conditions.
 bool quad_chunk_state_supported(const Params &p)
 {
