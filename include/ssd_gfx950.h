@@ -102,6 +102,11 @@ int ssd_state_passing_fwd(const ssd_tensor *states, const ssd_tensor *dA_chunk, 
  * initial_states is (b,H,P,N), out is (b,C,H,P,N), final_states is (b,H,P,N) f32, and the chunk-end decay
  * is read from dA_cumsum[..., Q-1].  states->data == NULL (or states == NULL) means "do not materialise the
  * per-chunk states"; otherwise they are written as a side effect exactly as ssd_chunk_state_fwd would.
+ * With few state tiles (batch * nheads * headdim / 32 below 512) and many chunks the call runs as a chunk-state launch
+ * that keeps every compute unit busy plus a streaming recurrence; that needs a place for the chunk states: a fp32
+ * `out` serves as one (the recurrence then works in place), and so does a fp32 `states` buffer.  With a 16-bit `out`
+ * and no `states` such a problem stays on the kernel with one workgroup per tile, which is slower (the library never
+ * allocates): a caller in that position gains by passing `states`.
  */
 int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
                                       const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
@@ -115,17 +120,6 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  * Pure host logic; launches nothing.
  */
 int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
-
-/*
- * No counterpart in the reference.  1 if ssd_fused_chunk_state_passing_fwd would finish sooner for these arguments
- * when it is handed a `states` buffer (fp32, (batch, nchunks, nheads, headdim, dstate), contiguous (headdim, dstate)
- * planes) than without one, 0 if not, negative = rejected.  That is the case for long sequences with few state tiles
- * (batch * nheads * headdim / 32 below 512): with the buffer the call runs as a chunk-state launch that keeps every
- * compute unit busy plus a streaming recurrence, without it on a kernel that has one workgroup per tile and walks
- * the chunks serially.  A caller that does not need the states may pass scratch memory; the library itself never
- * allocates.  Pure host logic; launches nothing.
- */
-int ssd_query_fused_wants_states(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
 
 /*
  * dt preparation and per-chunk cumulative sum, the producer of `dt` and `dA_cumsum` for the three calls above.

@@ -105,6 +105,15 @@ bool pair_supported(const Params &p)
     return ssd::quad_chunk_state_supported(cs);
 }
 
+// the fused call's arguments with `out` doubling as the `states` buffer
+Params with_states_in_out(const Params &p)
+{
+    Params q = p;
+    q.states = p.out; q.dt_states = p.dt_out;
+    q.sst_b = p.so_b; q.sst_c = p.so_c; q.sst_h = p.so_h; q.sst_p = p.so_p;
+    return q;
+}
+
 int run(const Params &p, bool fused, void *stream)
 {
     int rc = check_device();
@@ -117,8 +126,18 @@ int run(const Params &p, bool fused, void *stream)
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
     if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
-    else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8192)) &&
-             pair_supported(p)) {
+    else if (fused && !p.states && g_forced_split == 0 && tiles < 512 && (int64_t)tiles * p.C >= 8192 &&
+             p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p))) {
+        // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
+        // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
+        // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
+        const Params q = with_states_in_out(p);
+        Params cs = q;
+        cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
+        e = ssd::launch_quad_chunk_state(cs, s);
+        if (e == hipSuccess) e = ssd::launch_state_passing(pass_params_of(q), s);
+    } else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8192)) &&
+               pair_supported(p)) {
         // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
         // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
         // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
@@ -271,19 +290,6 @@ int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dim
     int rc = fill_common(p, x, B, &f32, &f32, nullptr, nullptr, dims, 1);
     if (rc) return rc;
     return ssd::mfma_supported(p) ? 1 : 0;
-}
-
-int ssd_query_fused_wants_states(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims)
-{
-    Params p;
-    ssd_tensor f32 = {(void *)16, SSD_F32, 0, {0, 0, 0, 1, 0}};
-    int rc = fill_common(p, x, B, &f32, &f32, nullptr, nullptr, dims, 1);
-    if (rc) return rc;
-    if (g_forced_split == 2 || g_forced_split == 4 || !ssd::quad_inputs_supported(p)) return 0;
-    const int tiles = p.batch * p.nheads * (p.headdim / 32);
-    if (g_forced_split == 1) return 0;                  // the fused four-tile kernel is forced and applies
-    if (tiles >= 512) return 0;                         // ... or chosen
-    return (int64_t)tiles * p.C >= 8192 ? 1 : 0;
 }
 
 int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *dt_out,

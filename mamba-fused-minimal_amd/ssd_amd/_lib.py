@@ -13,7 +13,7 @@ SSD_F32, SSD_BF16, SSD_F16 = 0, 1, 2
 _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_F16}
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
-           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_query_fused_wants_states", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
+           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
 class SsdTensor(ctypes.Structure):
@@ -53,8 +53,6 @@ def load():
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.argtypes = [T] * 11 + [D, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, vp]
     lib.ssd_query_path.restype = ctypes.c_int
     lib.ssd_query_path.argtypes = [T, T, D]
-    lib.ssd_query_fused_wants_states.restype = ctypes.c_int
-    lib.ssd_query_fused_wants_states.argtypes = [T, T, D]
     lib.ssd_chunk_cumsum_fwd.restype = ctypes.c_int
     lib.ssd_chunk_cumsum_fwd.argtypes = [T, T, T, T, T, i32, i32, i32, i32, ctypes.c_int, ctypes.c_float, ctypes.c_float, vp]
     lib.ssd_chunk_scan_states_fwd.restype = ctypes.c_int

@@ -130,10 +130,6 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     if initial_states is not None and initial_states.stride(-1) != 1:
         initial_states = initial_states.contiguous()
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
-    if states is None and lib.ssd_query_fused_wants_states(_lib.tensor_arg(x), _lib.tensor_arg(B), dims) == 1:
-        # few state tiles, many chunks: the library is faster with room for the per-chunk states (a chunk-state
-        # launch over every compute unit + the streaming recurrence); the buffer is scratch and dropped on return
-        states = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=torch.float32)
     with torch.cuda.device(x.device):
         rc = lib.ssd_fused_chunk_state_passing_fwd(
             _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),

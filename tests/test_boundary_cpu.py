@@ -83,24 +83,6 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_set_segment_chunks(-1) == -2 and lib.ssd_set_segment_chunks(3) == 0 and lib.ssd_set_segment_chunks(0) == 3
 
 
-def test_query_fused_wants_states(lib):
-    # few state tiles and many chunks: the fused call is faster with room for the per-chunk states; not so for
-    # short problems, for problems with at least 512 tiles (the fused four-tile kernel), or off the bf16 path
-    from ssd_amd import _lib
-    T = _lib.tensor_arg
-    def ask(b, L, H, P, N, G, Q, dtype=torch.bfloat16):
-        x = torch.empty(b, L, H, P, dtype=dtype)       # never read
-        B = torch.empty(b, L, G, N, dtype=dtype)
-        return lib.ssd_query_fused_wants_states(T(x), T(B), _lib.dims_arg(b, L, H, P, N, G, Q, -(-L // Q)))
-    assert ask(1, 65536, 8, 64, 128, 1, 128) == 1          # 16 tiles x 512 chunks
-    assert ask(1, 2048, 8, 64, 128, 1, 128) == 0           # 16 tiles x 16 chunks
-    assert ask(2, 4096, 128, 64, 128, 1, 256) == 0         # 512 tiles
-    assert ask(1, 65536, 8, 64, 128, 1, 128, torch.float32) == 0
-    assert ask(1, 65536, 8, 40, 128, 1, 128) == 0          # headdim 40: generic path
-    assert ask(1, 65536, 6, 64, 128, 2, 128) == 0          # six tiles per group: not a multiple of four
-    assert ask(1, 65536, 9, 64, 128, 2, 128) == -2         # nheads % ngroups
-
-
 def test_signatures_match_reference_call_surface():
     import ssd_amd
     sig = lambda f: list(inspect.signature(f).parameters)

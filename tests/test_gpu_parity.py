@@ -221,6 +221,21 @@ def test_chunk_state_segments(ops, oracle, kw, chunks):
         ops.set_segment_chunks(old_chunks)
 
 
+@pytest.mark.parametrize("kw", [
+    dict(L=65536, Q=128),                                # 16 tiles x 512 chunks
+    dict(L=70000, nseq=9, H=16, G=2),                    # ragged, packed sequences, grouped B: 32 tiles x 274 chunks
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_fused_few_tiles_many_chunks(ops, oracle, kw):
+    # fewer than 512 state tiles, at least 8192 tile-chunks, fp32 out, no states= buffer: the fused call runs as the
+    # chunk-state launch into `out` and the recurrence in place; with bf16 out it stays on the token-split kernel
+    base = dict(b=1, L=1024, H=8, G=1, init=True)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    _run_case(ops, oracle, d, with_states=False, check_unfused=False, name="in-place")
+    _run_case(ops, oracle, d, with_states=False, out_dtype=torch.bfloat16, check_unfused=False, name="in-place.bf16out")
+    _run_case(ops, oracle, d, with_states=True, check_unfused=False, name="with-states")
+
+
 def test_bf16_outputs(ops, oracle):
     d = oracle.make_inputs(1, b=2, L=1024, H=6, init=True)
     _run_case(ops, oracle, d, with_states=False, out_dtype=torch.bfloat16, check_unfused=False, name="bf16out")
