@@ -59,10 +59,18 @@ __global__ void __launch_bounds__(256) state_passing_kernel(const PassParams p)
     // `out` may be the buffer `states` lives in (slot c holds the chunk state of chunk c and receives the state that
     // enters chunk c): a lane only ever touches its own elements, reads slot c before it writes it, and memory
     // operations of one lane on one address keep their program order -- hence the first loads before the first store
+    // the chunk's decay and the id of its last token travel with its state: requested D chunks ahead as well
+    auto last_id = [&](int c) { return sq ? sq[(int64_t)(min((c + 1) * p.Q, p.seqlen) - 1) * p.ssq_l] : 0; };
     Vals<VEC> nxt[D];
+    float dan[D];
+    int32_t idn[D];
 #pragma unroll
     for (int i = 0; i < D; ++i)
-        if (i < p.C) nxt[i] = load_vals<VEC>(p.states, st_base + i * p.sst_c, p.dt_states);
+        if (i < p.C) {
+            nxt[i] = load_vals<VEC>(p.states, st_base + i * p.sst_c, p.dt_states);
+            dan[i] = da[i * p.sda_c];
+            idn[i] = last_id(i);
+        }
     store_vals<VEC>(p.out, out_base, p.dt_out, s);
     int32_t prev = 0;
     for (int c0 = 0; c0 < p.C; c0 += D) {
@@ -71,10 +79,14 @@ __global__ void __launch_bounds__(256) state_passing_kernel(const PassParams p)
             const int c = c0 + i;
             if (c < p.C) {
                 const Vals<VEC> cur = nxt[i];
-                if (c + D < p.C) nxt[i] = load_vals<VEC>(p.states, st_base + (int64_t)(c + D) * p.sst_c, p.dt_states);
-                float sc = __expf(da[c * p.sda_c]);
+                float sc = __expf(dan[i]);
+                const int32_t id = idn[i];
+                if (c + D < p.C) {
+                    nxt[i] = load_vals<VEC>(p.states, st_base + (int64_t)(c + D) * p.sst_c, p.dt_states);
+                    dan[i] = da[(c + D) * p.sda_c];
+                    idn[i] = last_id(c + D);
+                }
                 if (sq) {
-                    const int32_t id = sq[(int64_t)(min((c + 1) * p.Q, p.seqlen) - 1) * p.ssq_l];
                     if (id != prev) sc = 0.f;
                     prev = id;
                 }
