@@ -316,6 +316,7 @@ def test_reference_module_names_resolve(ops):
     dict(H=40, Q=128),                                   # two head tiles, the second partial
     dict(Q=1024, L=4096, b=1),                           # the largest chunk the kernel takes (> 64 KB of LDS)
     dict(dtype="fp32", b=1, L=1024),                     # fp32 dt
+    dict(dtype="fp16", b=1, L=512, H=8),                 # fp16 dt, half a head tile
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "base")
 def test_chunk_cumsum(ops, oracle, kw):
     base = dict(b=2, L=2048, H=24)
