@@ -157,9 +157,10 @@ int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tens
  * C: (batch, seqlen, ngroups, dstate); prev_states: (batch, nchunks, nheads, headdim, dstate), the `out` of the
  * state passing / fused calls above; dA_cumsum as above; seq_idx nullable; y: (batch, seqlen, nheads, headdim),
  * f32/bf16/f16.  Innermost strides of C, prev_states and y must be 1.  accumulate != 0 adds to what y holds (the
- * intra-chunk half of the scan computed elsewhere) instead of overwriting it.  bf16 C with fp32 states, dstate
- * 64/128, chunk size 64/128/256 and headdim % 32 == 0 run on the matrix cores with the fp32 state entering as
- * bf16 hi + lo (the reference rounds the state to C's element type); everything else on a plain FMA kernel.
+ * intra-chunk half of the scan computed elsewhere) instead of overwriting it.  bf16 C with fp32 or bf16 states,
+ * dstate 64/128, chunk size 64/128/256 and headdim % 32 == 0 run on the matrix cores: a fp32 state enters as bf16
+ * hi + lo (the reference rounds the state to C's element type), a bf16 state as it is; everything else on a plain
+ * FMA kernel.
  */
 int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states, const ssd_tensor *dA_cumsum,
                               const ssd_tensor *seq_idx, const ssd_tensor *y, const ssd_dims *dims, int accumulate,

@@ -96,17 +96,21 @@ __device__ __forceinline__ void store_y(__amdgpu_buffer_rsrc_t rsO, int dt_out, 
     }
 }
 
-template <int NK, int PB> constexpr int state_lds() { return PB * 16 * NK * 32 * 4; }          // rows x dstate fp32
+template <int NK, int PB, bool S16 = false> constexpr int state_lds() { return PB * 16 * NK * 32 * (S16 ? 2 : 4); }   // rows x dstate
 template <int NK, int PB> constexpr int wave_lds() { return 2 * 16 * NK * 32 * 2 + 16 * PB * 16 * 4; }   // 2 C blocks + y block
-template <int NK, int PB> constexpr int lds_bytes() { return state_lds<NK, PB>() + 4 * wave_lds<NK, PB>(); }
+template <int NK, int PB, bool S16 = false> constexpr int lds_bytes() { return state_lds<NK, PB, S16>() + 4 * wave_lds<NK, PB>(); }
 
 // NK = dstate / 32 (2 or 4); PB = headdim rows of the item / 16 (2 or 4); MB = 16-token blocks per wave = Q / 64;
-// PLAIN = y is fp32 and overwritten (the element-type and accumulate branches fold away).
-template <int NK, int PB, int MB, bool PLAIN>
+// PLAIN = y is fp32 and overwritten (the element-type and accumulate branches fold away);
+// S16 = the states are bf16 (what the reference hands its scan, kernels/ssd_chunk_scan.py:108): a row of the state is
+// an MFMA operand as it lies in memory -- half the bytes, no hi + lo split, half the MFMAs.
+template <int NK, int PB, int MB, bool PLAIN, bool S16>
 __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 {
     constexpr int N = 32 * NK;
-    constexpr int PRS = N / 4;          // 16-byte pieces per state row (fp32)
+    constexpr int SE = S16 ? 2 : 4;     // bytes per state element
+    constexpr int PRS = N * SE / 16;    // 16-byte pieces per state row
+    constexpr int SWZ = PRS < 16 ? PRS - 1 : 15;     // row bits XORed into the piece index of a state row in LDS
     constexpr int PRC = N / 8;          // 16-byte pieces per C row (bf16)
     constexpr int OP = PB * 4;          // 16-byte pieces per y row of the item (fp32)
     constexpr int SI = PB * 16 * PRS / 64 / 4;   // state load instructions per wave
@@ -115,7 +119,7 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
     const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     char *sld = lds;
-    char *cbuf = lds + state_lds<NK, PB>() + wave * wave_lds<NK, PB>();
+    char *cbuf = lds + state_lds<NK, PB, S16>() + wave * wave_lds<NK, PB>();
     char *obuf = cbuf + 2 * 16 * N * 2;
 
     // item -> (batch, chunk, head, row block): row blocks and heads vary fastest, so the workgroups in flight share
@@ -151,14 +155,14 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
     }
 
     // ---- requests: the state block (all waves together), then this wave's first two C blocks
-    const int64_t s_pitch = p.sst_p * 4;            // bytes
-    const auto rsS = make_rsrc((const char *)p.states + 4 * (b * p.sst_b + c * p.sst_c + h * p.sst_h + (int64_t)p0 * p.sst_p),
-                               (int64_t)(16 * PB - 1) * s_pitch + N * 4);
+    const int64_t s_pitch = p.sst_p * SE;           // bytes
+    const auto rsS = make_rsrc((const char *)p.states + SE * (b * p.sst_b + c * p.sst_c + h * p.sst_h + (int64_t)p0 * p.sst_p),
+                               (int64_t)(16 * PB - 1) * s_pitch + N * SE);
 #pragma unroll
     for (int i = 0; i < SI; ++i) {
         const int ins = wave * SI + i;                                  // covers LDS pieces 64 * ins .. + 63
         const int row = ins * (64 / PRS) + lane / PRS;
-        const int q = (lane % PRS) ^ (row & 15);
+        const int q = (lane % PRS) ^ (row & SWZ);
         load_to_lds(rsS, sld + ins * 1024, row * (int)s_pitch + q * 16, 0);
     }
     const int64_t c_pitch = p.sC_l * 2;
@@ -188,6 +192,11 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
     for (int j = 0; j < PB; ++j)
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks) {
+            if constexpr (S16) {
+                shi[j][ks] = *(const u32x4 *)(sld + (16 * j + i16) * (N * 2) + (((4 * ks + kg) ^ (i16 & SWZ)) << 4));
+                slo[j][ks] = (u32x4){0u, 0u, 0u, 0u};
+                continue;
+            }
             const int q0 = 8 * ks + 2 * kg;
             const char *rowp = sld + (16 * j + i16) * (N * 4);
             const f32x4 a = *(const f32x4 *)(rowp + ((q0 ^ i16) << 4));
@@ -241,11 +250,13 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 #pragma unroll
             for (int j = 0; j < PB; ++j)
                 acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[j][ks]), cf[ks], acc[j], 0, 0, 0);
+        if constexpr (!S16) {
 #pragma unroll
-        for (int ks = 0; ks < NK; ++ks)
+            for (int ks = 0; ks < NK; ++ks)
 #pragma unroll
-            for (int j = 0; j < PB; ++j)
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[j][ks]), cf[ks], acc[j], 0, 0, 0);
+                for (int j = 0; j < PB; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[j][ks]), cf[ks], acc[j], 0, 0, 0);
+        }
 
         // the C operands are in registers (the MFMAs above read them): the buffer can take block mb + 2
         __builtin_amdgcn_sched_barrier(0);
@@ -475,13 +486,13 @@ static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 
 bool scan_states_mfma_supported(const ScanParams &p)
 {
     using scan::aligned;
-    if (p.dt_C != DT_BF16 || p.dt_states != DT_F32) return false;
+    if (p.dt_C != DT_BF16 || (p.dt_states != DT_F32 && p.dt_states != DT_BF16)) return false;
     if (p.dstate != 64 && p.dstate != 128) return false;
     if (p.Q != 64 && p.Q != 128 && p.Q != 256) return false;
     if (p.headdim % 32 != 0) return false;
     if (!aligned(p.Cm, 16) || !aligned(p.states, 16) || !aligned(p.out, 16)) return false;
     if ((p.sC_b | p.sC_l | p.sC_g) % 8 != 0) return false;
-    if ((p.sst_b | p.sst_c | p.sst_h | p.sst_p) % 4 != 0) return false;
+    if ((p.sst_b | p.sst_c | p.sst_h | p.sst_p) % (p.dt_states == DT_F32 ? 4 : 8) != 0) return false;
     const int per16 = p.dt_out == DT_F32 ? 4 : 8;
     if ((p.so_b | p.so_l | p.so_h) % per16 != 0) return false;
     // byte offsets inside one descriptor are 32-bit
@@ -490,19 +501,19 @@ bool scan_states_mfma_supported(const ScanParams &p)
     return (int64_t)p.batch * p.C * p.nheads * (p.headdim / 32) < 0x7fffffffLL;
 }
 
-template <int NK, int PB, int MB, bool PLAIN>
+template <int NK, int PB, int MB, bool PLAIN, bool S16 = false>
 static hipError_t launch_scan_k(const ScanParams &p, hipStream_t s)
 {
-    constexpr int lds = scan::lds_bytes<NK, PB>();
+    constexpr int lds = scan::lds_bytes<NK, PB, S16>();
     static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
     if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_kernel<NK, PB, MB, PLAIN>,
+        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_kernel<NK, PB, MB, PLAIN, S16>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         configured = true;
     }
     const int64_t items = (int64_t)p.batch * p.C * p.nheads * (p.headdim / (16 * PB));
-    hipLaunchKernelGGL((scan::scan_states_kernel<NK, PB, MB, PLAIN>), dim3((unsigned)items), dim3(256), lds, s, p);
+    hipLaunchKernelGGL((scan::scan_states_kernel<NK, PB, MB, PLAIN, S16>), dim3((unsigned)items), dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
@@ -510,6 +521,13 @@ template <int NK, int PB>
 static hipError_t launch_scan_q(const ScanParams &p, hipStream_t s)
 {
     const bool plain = p.dt_out == DT_F32 && !p.accumulate;
+    if (p.dt_states == DT_BF16) {
+        switch (p.Q) {
+        case 64: return plain ? launch_scan_k<NK, PB, 1, true, true>(p, s) : launch_scan_k<NK, PB, 1, false, true>(p, s);
+        case 128: return plain ? launch_scan_k<NK, PB, 2, true, true>(p, s) : launch_scan_k<NK, PB, 2, false, true>(p, s);
+        default: return plain ? launch_scan_k<NK, PB, 4, true, true>(p, s) : launch_scan_k<NK, PB, 4, false, true>(p, s);
+        }
+    }
     switch (p.Q) {
     case 64: return plain ? launch_scan_k<NK, PB, 1, true>(p, s) : launch_scan_k<NK, PB, 1, false>(p, s);
     case 128: return plain ? launch_scan_k<NK, PB, 2, true>(p, s) : launch_scan_k<NK, PB, 2, false>(p, s);
@@ -551,7 +569,7 @@ int set_scan_kernel(int k)
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s)
 {
     if ((int64_t)p.batch * p.seqlen * p.nheads * p.headdim == 0) return hipSuccess;
-    if (scan_states_mfma_supported(p) && g_scan_kernel != 1 && p.headdim % 64 == 0 && p.sda_k == 1 &&
+    if (scan_states_mfma_supported(p) && p.dt_states == DT_F32 && g_scan_kernel != 1 && p.headdim % 64 == 0 && p.sda_k == 1 &&
         ((uintptr_t)p.dacs % 16) == 0 && (p.sda_b | p.sda_h | p.sda_c) % 4 == 0) {
         // runs of heads: the longest divisor of the heads per group up to 10 (enough workgroups to fill the chip
         // matter more than the last bit of C reuse)

@@ -437,6 +437,16 @@ def _scan_states_case(ops, oracle, base):
     torch.cuda.synchronize()
     assert got.data_ptr() == view.data_ptr()
     _check("scan_states.accumulate", view, want + wide[..., 8:])
+    # bf16 passed states (what the reference's scan is handed, main.py:85-100): judged against the oracle on the same
+    # rounded states -- the kernel then does what the fp32 one does, minus the rounding of its own hi + lo split
+    prev16 = prev.to(torch.bfloat16)
+    want16 = oracle.chunk_scan_states_ref(C, prev16.float(), dA, seq_idx=seq)
+    y16 = ops._chunk_scan_states_fwd(Cd, _dev(prev16), dAd, seq_idx=sd, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    _check("scan_states.bf16states", y16, want16)
+    got = ops._chunk_scan_states_fwd(Cd, _dev(prev16), dAd, seq_idx=sd, out=view, accumulate=True)
+    torch.cuda.synchronize()
+    _check("scan_states.bf16states.accumulate", view, want + want16 + wide[..., 8:], 2e-3, 2e-3)
 
 
 def test_chunk_scan_states_cfg2_row(ops, oracle):
