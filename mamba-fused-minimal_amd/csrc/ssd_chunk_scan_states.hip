@@ -96,6 +96,34 @@ __device__ __forceinline__ void store_y(__amdgpu_buffer_rsrc_t rsO, int dt_out, 
     }
 }
 
+// Eight consecutive values of one y row as 16-bit elements: one 16-byte store (and load, when accumulating).
+__device__ __forceinline__ void store_y8(__amdgpu_buffer_rsrc_t rsO, int dt_out, int accumulate, int voff, int soff, f32x4 a, f32x4 d)
+{
+    const bool bf = dt_out == DT_BF16;
+    float v[8] = {a.x, a.y, a.z, a.w, d.x, d.y, d.z, d.w};
+    if (accumulate) {
+        const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(rsO, 2 * voff, 2 * soff, 0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t w = (e & 1) ? (o[e >> 1] >> 16) : (o[e >> 1] & 0xffffu);
+            v[e] += bf ? bf16_bits_to_f32(w) : (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+        }
+    }
+    u32x4 q;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (bf) {
+            q[e] = pack_bf16(v[2 * e], v[2 * e + 1]);
+        } else {
+            typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+            const h2 t = {(_Float16)v[2 * e], (_Float16)v[2 * e + 1]};
+            q[e] = __builtin_bit_cast(uint32_t, t);
+        }
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(q, rsO, 2 * voff, 2 * soff, 0);
+    asm volatile("s_nop 3" ::"v"(q) : "memory");
+}
+
 template <int NK, int PB, bool S16 = false> constexpr int state_lds() { return PB * 16 * NK * 32 * (S16 ? 2 : 4); }   // rows x dstate
 template <int NK, int PB> constexpr int wave_lds() { return 2 * 16 * NK * 32 * 2 + 16 * PB * 16 * 4; }   // 2 C blocks + y block
 template <int NK, int PB, bool S16 = false> constexpr int lds_bytes() { return state_lds<NK, PB, S16>() + 4 * wave_lds<NK, PB>(); }
@@ -223,7 +251,8 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         // C block mb has landed once no more operations are outstanding than were issued behind its requests
-        constexpr int kNext = CI, kSt = PB;
+        // (a 16-bit y leaves as PB / 2 stores of 16 bytes; counting fewer operations than were issued is safe)
+        constexpr int kNext = CI, kSt = PLAIN ? PB : PB / 2;
         const int behind = mb == 0 ? (MB > 1 ? kNext : 0)
                          : mb == 1 ? (MB > 2 ? kNext : 0) + kSt
                                    : kSt + (mb + 1 < MB ? kNext : 0) + kSt;
@@ -267,6 +296,23 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 #pragma unroll
         for (int j = 0; j < PB; ++j)
             *(f32x4 *)(obuf + i16 * (OP * 16) + ((((4 * j + kg) ^ i16) & (OP - 1)) << 4)) = acc[j] * sc[mb];
+        if (!PLAIN && p.dt_out != DT_F32) {
+            // 16-bit y: a lane takes two adjacent pieces of a token row, eight values, and stores 16 bytes
+            constexpr int OP2 = OP / 2;
+            f32x4 ya[PB / 2], yd[PB / 2];
+#pragma unroll
+            for (int r = 0; r < PB / 2; ++r) {
+                const int t = r * (64 / OP2) + lane / OP2, pp = lane % OP2;
+                ya[r] = *(const f32x4 *)(obuf + t * (OP * 16) + ((((2 * pp) ^ t) & (OP - 1)) << 4));
+                yd[r] = *(const f32x4 *)(obuf + t * (OP * 16) + ((((2 * pp + 1) ^ t) & (OP - 1)) << 4));
+            }
+#pragma unroll
+            for (int r = 0; r < PB / 2; ++r) {
+                const int t = r * (64 / OP2) + lane / OP2, pp = lane % OP2;
+                store_y8(rsO, p.dt_out, p.accumulate, t * (int)o_pitch + 8 * pp, (tok0 + 16 * mb) * (int)o_pitch, ya[r], yd[r]);
+            }
+            continue;
+        }
         f32x4 yv[PB];
 #pragma unroll
         for (int r = 0; r < PB; ++r) {
