@@ -105,6 +105,15 @@ bool pair_supported(const Params &p)
     return ssd::quad_chunk_state_supported(cs);
 }
 
+// chunk states into p.states, then the recurrence over them into p.out / p.fin (which may be the same buffer)
+hipError_t launch_pair(const Params &p, hipStream_t s)
+{
+    Params cs = p;
+    cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
+    const hipError_t e = ssd::launch_quad_chunk_state(cs, s);
+    return e == hipSuccess ? ssd::launch_state_passing(pass_params_of(p), s) : e;
+}
+
 // the fused call's arguments with `out` doubling as the `states` buffer
 Params with_states_in_out(const Params &p)
 {
@@ -131,22 +140,14 @@ int run(const Params &p, bool fused, void *stream)
         // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
         // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
         // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
-        const Params q = with_states_in_out(p);
-        Params cs = q;
-        cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
-        e = ssd::launch_quad_chunk_state(cs, s);
-        if (e == hipSuccess) e = ssd::launch_state_passing(pass_params_of(q), s);
+        e = launch_pair(with_states_in_out(p), s);
     } else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8192)) &&
                pair_supported(p)) {
         // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
         // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
         // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
-        Params cs = p;
-        cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
-        e = ssd::launch_quad_chunk_state(cs, s);
-        if (e == hipSuccess) e = ssd::launch_state_passing(pass_params_of(p), s);
-    }
-    else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 2048)) &&
+        e = launch_pair(p, s);
+    } else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 2048)) &&
              ssd::quad_chunk_state_supported(p))
         e = ssd::launch_quad_chunk_state(p, s);
     else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
