@@ -236,6 +236,30 @@ def test_fused_few_tiles_many_chunks(ops, oracle, kw):
     _run_case(ops, oracle, d, with_states=True, check_unfused=False, name="with-states")
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_shapes_through_the_dispatcher(ops, oracle, seed):
+    # seeded random draws over shapes and options, each run with the library choosing the kernels by itself and with
+    # the four-tile kernel forced: whatever path the dispatcher takes, the results are the oracle's
+    import random
+    rng = random.Random(1000 + seed)
+    P = rng.choice([32, 64, 128])
+    G = rng.choice([1, 2])
+    H = G * rng.choice([2, 4, 6])
+    Q = rng.choice([128, 256])
+    kw = dict(b=rng.choice([1, 2, 3]), H=H, G=G, P=P, N=rng.choice([64, 128]), Q=Q,
+              L=rng.choice([Q, 3 * Q + 17, 5 * Q, 9 * Q - 1]), nseq=rng.choice([0, 0, 3]), init=rng.random() < 0.5)
+    d = oracle.make_inputs(1, **kw)
+    with_states = rng.random() < 0.5
+    lowp = rng.random() < 0.3
+    for forced in (0, 1):
+        old = ops.set_token_split(forced)
+        try:
+            _run_case(ops, oracle, d, with_states=with_states and not lowp, out_dtype=torch.bfloat16 if lowp else torch.float32,
+                      check_unfused=not lowp, name=f"random{seed}.split{forced}")
+        finally:
+            ops.set_token_split(old)
+
+
 def test_bf16_outputs(ops, oracle):
     d = oracle.make_inputs(1, b=2, L=1024, H=6, init=True)
     _run_case(ops, oracle, d, with_states=False, out_dtype=torch.bfloat16, check_unfused=False, name="bf16out")
