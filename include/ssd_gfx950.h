@@ -178,8 +178,9 @@ int ssd_set_scan_kernel(int kernel);
  * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
  * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
  * waves per state tile; 1 = one wave per state tile (the kernel with four tiles per workgroup) wherever that
- * kernel applies.  The setting holds for every later call of this process.  Returns the previous setting, or
- * SSD_ERR_SHAPE for any other value.  Results agree between the settings to rounding (the tokens are summed in
+ * kernel applies; 3 = the fused kernel with three tiles per workgroup whose four waves each take two of a chunk's
+ * eight steps for all three tiles (dstate 128, chunk 256, fp32 states; the library never picks it by itself).  The setting holds for every later call of this process.  Returns the previous setting, or
+ * SSD_ERR_SHAPE for a value outside 0..4.  Results agree between the settings to rounding (the tokens are summed in
  * another order), not bit for bit.
  */
 int ssd_set_token_split(int waves);

@@ -133,7 +133,9 @@ int run(const Params &p, bool fused, void *stream)
     // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
     // kernel, which puts four waves on every tile, has the shorter chunk.
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
-    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
+    if (fused && g_forced_split == 3 && ssd::step_split_supported(p))
+        e = ssd::launch_step_split(p, s);       // never chosen by itself: slower than the four-tile kernel so far
+    else if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
     else if (fused && !p.states && g_forced_split == 0 && tiles < 512 && (int64_t)tiles * p.C >= 8192 &&
              p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p))) {
@@ -373,10 +375,10 @@ int ssd_set_segment_chunks(int chunks)
 
 int ssd_set_token_split(int waves)
 {
-    if (waves != 0 && waves != 1 && waves != 2 && waves != 4) return SSD_ERR_SHAPE;
+    if (waves < 0 || waves > 4) return SSD_ERR_SHAPE;
     const int old = g_forced_split;
     g_forced_split = waves;
-    ssd::set_token_split(waves == 1 ? 0 : waves);
+    ssd::set_token_split(waves == 2 || waves == 4 ? waves : 0);
     return old;
 }
 

@@ -135,6 +135,8 @@ hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
 hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state tiles per workgroup sharing B in LDS
 bool quad_supported(const Params &p);
+hipError_t launch_step_split(const Params &p, hipStream_t s);   // fused: three tiles per workgroup, steps dealt to the waves
+bool step_split_supported(const Params &p);
 hipError_t launch_quad_chunk_state(const Params &p, hipStream_t s);     // chunk states only, same kernel
 bool quad_chunk_state_supported(const Params &p);
 bool quad_inputs_supported(const Params &p);     // what the four-tile kernel asks of x, B, dt, dA_cumsum and the shape

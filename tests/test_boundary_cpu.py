@@ -79,7 +79,7 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA), T(None), T(y), bad, 0, None) == -2
     assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA.bfloat16()), T(None), T(y), dims, 0, None) == -3
     assert lib.ssd_chunk_scan_states_fwd(T(Cm), T(st), T(dA), T(None), T(y.transpose(2, 3)), dims, 0, None) == -4
-    assert lib.ssd_set_token_split(3) == -2 and lib.ssd_set_token_split(1) == 0 and lib.ssd_set_token_split(0) == 1
+    assert lib.ssd_set_token_split(5) == -2 and lib.ssd_set_token_split(1) == 0 and lib.ssd_set_token_split(0) == 1
     assert lib.ssd_set_segment_chunks(-1) == -2 and lib.ssd_set_segment_chunks(3) == 0 and lib.ssd_set_segment_chunks(0) == 3
 
 
