@@ -47,7 +47,8 @@ typedef enum ssd_status {
     SSD_ERR_DTYPE = -3,       /* element type not supported for this argument */
     SSD_ERR_STRIDE = -4,      /* innermost stride != 1 where the kernels need it */
     SSD_ERR_DEVICE = -5,      /* current device is not gfx950, or no device */
-    SSD_ERR_SCRATCH = -6      /* internal scratch could not be obtained */
+    SSD_ERR_SCRATCH = -6,     /* a kernel was asked for that needs a workspace, and none (or too small a one) was given */
+    SSD_ERR_CHAIN_TIMEOUT = -7 /* reported by ssd_fused_workspace_status: a bounded flag wait ran out */
 } ssd_status;
 
 /* A strided device tensor.  stride[i] is in elements; unused trailing entries are ignored. */
@@ -115,6 +116,53 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
                                       const ssd_dims *dims, int clamp, void *stream);
 
 /*
+ * The fused call with a caller-provided workspace, which opens the kernel that spreads ONE sequence's chunks over
+ * all compute units.  The reference does the same job with scratch tensors it allocates per call: two ticket
+ * counters and a global barrier (kernels/fused_globalbar.py:130-137, 237-238), or per-(batch, head) completion
+ * counters plus a throttle semaphore (kernels/fused_concurrent.py:81-84, 141, 205-208, 296-298).  Here work items
+ * (four state tiles sharing B x one chunk) are drawn from a device-wide ticket counter in chunk-major order; an
+ * item accumulates its chunk state from zero, then waits for the flag of the state entering its chunk, reads that
+ * state back from `out`, adds exp(dA_chunk) [same sequence] times it, stores the result as the next passed state
+ * and raises the next flag.  An item only waits for an item with a smaller ticket and tickets are drawn by running
+ * workgroups only, so the chain makes progress whatever workgroups are resident.  The wait is bounded nevertheless
+ * (spin_limit polls): a wave that gives up sets the error word of the workspace and still raises its own flag, so
+ * the launch always drains; ssd_fused_workspace_status reports it.
+ *
+ * workspace: device memory, 4-byte aligned, at least ssd_fused_workspace_bytes(dims); the call clears what it uses
+ * (a small fill launch, no memset node), so the memory may hold anything and may be reused by later calls on the
+ * same stream.  Two calls whose kernels may overlap (different streams) need workspaces of their own.
+ * kernel: SSD_KERNEL_AUTO lets the library choose between this kernel and those of ssd_fused_chunk_state_passing_fwd
+ * (which it runs when the shape, element types or a `states` output rule the chain kernel out: it needs bf16 x / B,
+ * fp32 out / initial / final states, no `states`, dstate 64 or 128, chunk 128 or 256); SSD_KERNEL_CHAIN insists on it
+ * and returns SSD_ERR_SCRATCH where it cannot run.  opts == NULL behaves as ssd_fused_chunk_state_passing_fwd.
+ */
+typedef struct ssd_fused_opts {
+    void *workspace;
+    uint64_t workspace_bytes;
+    int32_t spin_limit;       /* flag polls before a wave gives up; 0 = default (about 4 million) */
+    int32_t kernel;           /* SSD_KERNEL_AUTO, or one of the SSD_KERNEL_CHAIN values to insist on that kernel */
+    int32_t chunks_per_item;  /* chain kernel: consecutive chunks per work item, 1, 2 or 4; 0 = choose */
+    int32_t reserved;
+} ssd_fused_opts;
+
+enum { SSD_KERNEL_AUTO = 0, SSD_KERNEL_CHAIN = 1, SSD_KERNEL_CHAIN_LOCAL = 2, SSD_KERNEL_CHAIN_GLOBAL = 3 };
+
+uint64_t ssd_fused_workspace_bytes(const ssd_dims *dims);
+
+int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                         const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                         const ssd_tensor *initial_states, const ssd_tensor *states,
+                                         const ssd_tensor *out, const ssd_tensor *final_states,
+                                         const ssd_dims *dims, int clamp, const ssd_fused_opts *opts, void *stream);
+
+/*
+ * Waits for `stream` and reads the error word of a workspace used by ssd_fused_chunk_state_passing_fwd_ws:
+ * SSD_OK, or SSD_ERR_CHAIN_TIMEOUT when a wave of the last launch gave up waiting (the outputs are then unusable).
+ * No counterpart in the reference, whose spin loops are unbounded (kernels/fused_concurrent.py:11, 300).
+ */
+int ssd_fused_workspace_status(const void *workspace, void *stream);
+
+/*
  * Which kernel family the three calls above would pick for these arguments: 1 = bf16 MFMA path,
  * 0 = generic FMA path (other element types or shapes the MFMA tiling does not cover), negative = rejected.
  * Pure host logic; launches nothing.
@@ -178,9 +226,11 @@ int ssd_set_scan_kernel(int kernel);
  * Tuning / test hook with no counterpart in the reference: which bf16 MFMA kernel family serves the calls above.
  * 0 = let the library choose from the problem size (the default); 2 or 4 = the token-split kernels with that many
  * waves per state tile; 1 = one wave per state tile (the kernel with four tiles per workgroup) wherever that
- * kernel applies; 3 = the fused kernel with three tiles per workgroup whose four waves each take two of a chunk's
- * eight steps for all three tiles (dstate 128, chunk 256, fp32 states; the library never picks it by itself).  The setting holds for every later call of this process.  Returns the previous setting, or
- * SSD_ERR_SHAPE for a value outside 0..4.  Results agree between the settings to rounding (the tokens are summed in
+ * kernel applies.  While the setting is not 0 the library does not pick the ticket / flag-chain kernel by itself either
+ * (ssd_fused_chunk_state_passing_fwd_ws).  A process-wide hook for tests and tuning: it is atomic, so changing it while
+ * another thread launches is safe, but that thread's choice of kernel is then either the old or the new one.  The
+ * setting holds for every later call of this process.  Returns the previous setting, or
+ * SSD_ERR_SHAPE for a value other than 0, 1, 2, 4.  Results agree between the settings to rounding (the tokens are summed in
  * another order), not bit for bit.
  */
 int ssd_set_token_split(int waves);

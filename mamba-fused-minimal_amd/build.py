@@ -10,7 +10,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libssd_gfx950.so")
-SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_step_split.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip"]
+OBJ_DIR = os.path.join(HERE, "build")
+SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_chain.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # keep the compiler from forming packed-fp32 VALU instructions
@@ -26,17 +27,38 @@ def hipcc():
     return exe
 
 
-def build_library(verbose=False, extra_flags=()):
-    cmd = [hipcc(), *FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB]
-    if verbose:
-        print(" ".join(cmd))
+def _run(cmd):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"
     out = "\n".join(l for l in res.stdout.splitlines() if noise not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + out)
+    return out
+
+
+def build_library(verbose=False, extra_flags=(), jobs=None):
+    """Compiles every source to an object (in parallel: the files are independent) and links the shared library."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 8)
+
+    def compile_one(src):
+        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc(), *compile_flags, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd))
+        return obj, _run(cmd)
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(compile_one, SOURCES))
+    out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in results], "-o", LIB])
+    if verbose:
+        for _, text in results:
+            if text.strip():
+                print(text)
+        if out.strip():
+            print(out)
     return LIB
 
 

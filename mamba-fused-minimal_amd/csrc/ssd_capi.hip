@@ -5,28 +5,43 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+
 namespace {
 
 using ssd::Params;
 using ssd::PassParams;
 
-int g_forced_split = 0;     // ssd_set_token_split: 0 = choose, 1 = four-tile kernel, 2 / 4 = token-split kernels
+// ssd_set_token_split: 0 = choose, 1 = four-tile kernel, 2 / 4 = token-split kernels.  A process-wide test and tuning
+// hook: atomic, so that setting it while another thread launches is a race on the choice only, never on memory.
+std::atomic<int> g_forced_split{0};
 
 bool dtype_ok(int dt) { return dt == SSD_F32 || dt == SSD_BF16 || dt == SSD_F16; }
 
-// Device check, cached per device ordinal: the kernels are gfx950 code objects only.
-int check_device()
+// Device check, cached per device ordinal: the kernels are gfx950 code objects only.  A cache entry is written
+// once with its final value (0 = unknown, else 1 = gfx950 / 2 = another device, plus the compute-unit count
+// shifted left by 8), so concurrent first calls at worst query the device twice.
+std::atomic<int> g_device_cache[64];
+
+int device_info()
 {
-    static int cached[64];      // 0 = unknown, 1 = ok, 2 = not gfx950
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0) return SSD_ERR_DEVICE;
-    if (dev < 64 && cached[dev]) return cached[dev] == 1 ? SSD_OK : SSD_ERR_DEVICE;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) return 0;
+    if (dev < 64) {
+        const int c = g_device_cache[dev].load(std::memory_order_acquire);
+        if (c) return c;
+    }
     hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return SSD_ERR_DEVICE;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
     const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-    if (dev < 64) cached[dev] = ok ? 1 : 2;
-    return ok ? SSD_OK : SSD_ERR_DEVICE;
+    const int c = (ok ? 1 : 2) | (prop.multiProcessorCount << 8);
+    if (dev < 64) g_device_cache[dev].store(c, std::memory_order_release);
+    return c;
 }
+
+int check_device() { return (device_info() & 255) == 1 ? SSD_OK : SSD_ERR_DEVICE; }
+
+int compute_units() { return device_info() >> 8; }
 
 int check_dims(const ssd_dims *d)
 {
@@ -133,9 +148,8 @@ int run(const Params &p, bool fused, void *stream)
     // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
     // kernel, which puts four waves on every tile, has the shorter chunk.
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
-    if (fused && g_forced_split == 3 && ssd::step_split_supported(p))
-        e = ssd::launch_step_split(p, s);       // never chosen by itself: slower than the four-tile kernel so far
-    else if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
+    const int g_forced_split = ::g_forced_split.load(std::memory_order_relaxed);      // one value for the whole choice
+    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
     else if (fused && !p.states && g_forced_split == 0 && tiles < 512 && (int64_t)tiles * p.C >= 8192 &&
              p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p))) {
@@ -156,6 +170,15 @@ int run(const Params &p, bool fused, void *stream)
     return (int)e;
 }
 
+// Whether the ticket / flag-chain kernel is the better fused kernel for a problem it covers: it keeps every compute
+// unit busy whatever the number of state tiles, at the price of reading each passed state back once.
+bool chain_preferred(const Params &p)
+{
+    // it needs several items of four chunks per compute unit to pay for its start and its chain
+    const int64_t units = (int64_t)p.batch * p.nheads * (p.headdim / 32) / 4;
+    return p.C >= 16 && units * (p.C / 4) >= 3 * (int64_t)compute_units();
+}
+
 }  // namespace
 
 extern "C" {
@@ -171,7 +194,8 @@ const char *ssd_status_string(int status)
         case SSD_ERR_DTYPE: return "unsupported element type";
         case SSD_ERR_STRIDE: return "innermost stride must be 1";
         case SSD_ERR_DEVICE: return "no gfx950 device is current";
-        case SSD_ERR_SCRATCH: return "internal scratch unavailable";
+        case SSD_ERR_SCRATCH: return "workspace missing or too small for the requested kernel";
+        case SSD_ERR_CHAIN_TIMEOUT: return "a wave of the flag-chain kernel gave up waiting for its predecessor";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -222,6 +246,50 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
     int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, states, out, final_states, dims, clamp);
     if (rc) return rc;
     return run(p, true, stream);
+}
+
+uint64_t ssd_fused_workspace_bytes(const ssd_dims *dims)
+{
+    if (check_dims(dims)) return 0;
+    return ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+}
+
+int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                         const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                         const ssd_tensor *initial_states, const ssd_tensor *states,
+                                         const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims,
+                                         int clamp, const ssd_fused_opts *opts, void *stream)
+{
+    Params p;
+    int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, states, out, final_states, dims, clamp);
+    if (rc) return rc;
+    const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
+    if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
+    const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
+                         opts->workspace_bytes >= ssd_fused_workspace_bytes(dims);
+    if (have_ws && ssd::chain_supported(p) && (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p)))) {
+        rc = check_device();
+        if (rc) return rc;
+        p.ws = (int *)opts->workspace;
+        p.spin_limit = opts->spin_limit;
+        p.n_seg = opts->chunks_per_item == 1 || opts->chunks_per_item == 2 || opts->chunks_per_item == 4 ? opts->chunks_per_item : 0;
+        return (int)ssd::launch_chain(p, compute_units(), kernel == SSD_KERNEL_CHAIN_LOCAL ? 1 : kernel == SSD_KERNEL_CHAIN_GLOBAL ? 2 : 0,
+                                      (hipStream_t)stream);
+    }
+    if (kernel != SSD_KERNEL_AUTO) return SSD_ERR_SCRATCH;     // forced, but no workspace or not a shape it covers
+    return run(p, true, stream);
+}
+
+int ssd_fused_workspace_status(const void *workspace, void *stream)
+{
+    if (!workspace) return SSD_ERR_NULL;
+    int rc = check_device();
+    if (rc) return rc;
+    int word = 0;       // the error word sits behind the sixteen ticket counters
+    hipError_t e = hipMemcpyAsync(&word, (const int *)workspace + 16, sizeof(word), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return (int)e;
+    return word ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
 }
 
 int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
@@ -375,9 +443,8 @@ int ssd_set_segment_chunks(int chunks)
 
 int ssd_set_token_split(int waves)
 {
-    if (waves < 0 || waves > 4) return SSD_ERR_SHAPE;
-    const int old = g_forced_split;
-    g_forced_split = waves;
+    if (waves < 0 || waves > 4 || waves == 3) return SSD_ERR_SHAPE;
+    const int old = g_forced_split.exchange(waves);
     ssd::set_token_split(waves == 2 || waves == 4 ? waves : 0);
     return old;
 }

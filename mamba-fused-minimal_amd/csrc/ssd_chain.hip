@@ -1,0 +1,702 @@
+// Fused chunk-state + state-passing kernel whose work is handed out by tickets and ordered by a flag chain (gfx950).
+//
+// Why: a compute unit's vector-memory pipe takes loads and stores one after the other (moving this path's bytes
+// alone, with no arithmetic, takes 163 us on the 160 compute units that b=4 L=8192 H=80 fills when every state tile
+// stays on one compute unit for the whole sequence), so every compute unit has to carry its share of the traffic
+// whatever the number of tiles.  That means cutting a sequence's chunks loose from each other:
+//
+// A work item is R consecutive chunks of one unit, a unit being four state tiles -- (batch, head, 32 headdim rows) x
+// all of dstate, one per wave -- that share (batch, group) and therefore B.  Persistent workgroups, one per compute
+// unit, draw items from a ticket counter in chunk-major order (ticket t -> chunks R (t / units) ..., unit t % units),
+// so an item only ever depends on an item with a smaller ticket:
+//   1. each chunk state S_c = sum_k B_k (x w)_k (kernels/ssd_chunk_state.py:134-173) is accumulated from zero in the
+//      MFMA accumulators, independent of every other chunk, and parked in registers (R tiles of 64 per lane);
+//   2. the wave then waits for the flag of (tile, first chunk), which says that out[:, c0] -- the state entering the
+//      item -- is complete, reads it back, runs s_{c+1} = exp(dA_c) [same sequence] s_c + S_c
+//      (kernels/ssd_state_passing.py:69-84) over its R chunks in registers, stores the last state first, raises the
+//      flag of (tile, c0 + R) once that store is acknowledged, and stores the other R - 1 states after that.  Chunk 0
+//      starts from initial_states (or zero) and also writes out[:, 0]; an item whose first decay is zero (a sequence
+//      boundary) neither waits nor reads.
+// A link of the chain costs a few memory round trips (8 us measured under load); with R chunks per item there are
+// C / R links per sequence, consecutive items of a unit start R times further apart than with single chunks, and
+// only every R-th passed state is read back.
+// This chain replaces the reference's global barrier between its two phases (kernels/fused_globalbar.py:130-137)
+// and its per-(batch, head) completion counters with a throttle semaphore (kernels/fused_concurrent.py:81-84, 141,
+// 205-208).  It cannot deadlock and assumes nothing about which workgroups are resident: tickets are only drawn by
+// running workgroups, a workgroup finishes its items in ticket order, and the unfinished item with the smallest
+// ticket never waits for an unfinished one.  The wait is bounded all the same: after p.spin_limit polls a wave sets
+// the error word of the workspace, goes on with whatever out[:, c0] holds and still raises its flag, so that every
+// workgroup drains and the host can report the failure.
+//
+// Data movement inside a chunk is that of the four-tiles-per-workgroup kernel (ssd_quad.hip): B once per workgroup
+// through a four-step LDS ring read back with transposing loads, x rows through a per-wave ring, bf16 hi + lo
+// operands, all requests three steps ahead -- across chunk and item boundaries: the ticket of the next item is known
+// while an item runs, so the first steps of the next chunk are always on their way when the current one ends.
+#include "ssd_tile.h"
+
+namespace ssd {
+
+namespace chain {
+
+using namespace tile;
+
+// steps of B and x kept in LDS (requested ring - 1 steps ahead): 8 where a chunk has 8 steps -- one workgroup per
+// compute unit leaves the room, and the burst of state stores that ends an item drains behind requests that far
+// ahead -- else 4
+template <int SPC> constexpr int ring_of() { return SPC >= 8 ? 8 : 4; }
+// per wave: x ring + two weight slots (the next item's weights are written while the current item's are in use)
+template <int SPC> constexpr int wave_lds() { return ring_of<SPC>() * 2048 + 2 * 32 * SPC * 4; }
+constexpr int kStage = 1024;        // per wave: a 16 x 16 fp32 block of the state on its way to or from memory
+constexpr int kTicketBytes = 64;
+template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * NT * 1024 + 4 * (wave_lds<SPC>() + kStage) + kTicketBytes; }
+
+// How the passed states cross between compute units.  The L2 caches, one per XCD (32 compute units), are not
+// coherent with each other, and a device-scope release / acquire pair writes back and invalidates a whole L2
+// (measured: 1.2 ms per launch at b=4 L=8192 H=80 -- unusable).  Two ways remain, chosen per launch:
+//  * LOCAL: every unit belongs to one XCD.  Each XCD has its own ticket counter over its own units, a workgroup reads
+//    the id of the XCD it runs on from the hardware and draws from that counter, so producer and consumer of a passed
+//    state always share an L2: plain stores (written through the per-CU cache into L2), the flag raised once they
+//    have been acknowledged, flag polls that miss the per-CU cache (sc1), and plain read-back loads -- a compute unit
+//    reads each out[:, c] once, so its own cache cannot hold an older copy.  A link of the chain costs L2 latencies.
+//  * GLOBAL (few units, or units that do not spread evenly over the XCDs): one counter; the state stores, the
+//    read-back loads and the flags carry the device-scope cache policy (sc1: written through to memory, read around
+//    the L2), nothing is flushed.  A link costs memory latencies (about 9 us measured).
+constexpr int kAuxDevice = 16;      // sc1
+constexpr int kMaxXcd = 16;
+
+// workspace: [0..15] ticket counters (one per XCD slot), [16] error word, [32..47] hardware id of the XCD that
+// took each slot (+1), flags from [kWsHeaderInts]
+constexpr int kWsHeaderInts = 64, kWsErr = 16, kWsOwner = 32;
+
+// NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (4 or 8); R = chunks per work item (1, 2 or 4).
+// out, initial_states and final_states are fp32.
+template <int NT, int SPC, int R, bool HAS_SEQ, bool LOCAL>
+__global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
+{
+    constexpr int Q = 32 * SPC;
+    constexpr int kRing = ring_of<SPC>(), kDist = kRing - 1;
+    static_assert(kDist < SPC, "the requests of a step reach into the next chunk at most");
+    constexpr int TPL = Q / 64;         // tokens per lane when an item's weights are computed (2 or 4)
+    constexpr int NTW = NT / 4;         // B tile blocks (32 tokens x 16 columns, 1 KB) a wave fetches per step
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    char *bring = lds;                                                   // kRing x NT blocks of 1 KB, shared
+    char *xring = lds + kRing * NT * 1024 + wave * wave_lds<SPC>();      // kRing slots x (32 tokens x 64 bytes)
+    char *wbuf = xring + kRing * 2048;                                   // 2 slots x Q weights
+    char *stage = lds + kRing * NT * 1024 + 4 * wave_lds<SPC>() + wave * kStage;
+#if defined(__HIP_DEVICE_COMPILE__)      // typed as LDS: a volatile access through a generic pointer would go the flat way
+    typedef __attribute__((address_space(3))) volatile int lds_int;
+    lds_int *tq = (lds_int *)(__attribute__((address_space(3))) char *)(lds + lds_bytes<NT, SPC>() - kTicketBytes);
+#else
+    volatile int *tq = (volatile int *)(lds + lds_bytes<NT, SPC>() - kTicketBytes);
+#endif
+
+    constexpr int kAux = LOCAL ? 0 : kAuxDevice;
+    // this workgroup's share of the units: all of them, or those of the XCD it runs on (contiguous ranges)
+    int xcd_hw = 0, slot = 0, unit0 = 0, n_units = p.n_items >> 2;
+    if (LOCAL) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        xcd_hw = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;       // XCC_ID, bits 3:0
+#endif
+        slot = xcd_hw % p.n_xcd;
+        const int base = n_units / p.n_xcd, rem = n_units % p.n_xcd;
+        unit0 = slot * base + min(slot, rem);
+        n_units = base + (slot < rem ? 1 : 0);
+    }
+    const int n_super = (p.C + R - 1) / R;      // items per unit
+    const int total = n_units * n_super;
+    const int n_pt = p.headdim >> 5;
+    const int L = p.seqlen, C = p.C;
+    const int64_t xrb = 2 * p.sx_l, Brb = 2 * p.sB_l;            // row pitch in bytes
+    int *const ws_ticket = p.ws + slot, *const ws_err = p.ws + kWsErr, *const ws_flags = p.ws + kWsHeaderInts;
+
+    // ---- work items ------------------------------------------------------------------------------------------
+    // A workgroup walks a stream of chunks: the R chunks of its current item, then those of the next.  `Item` is one
+    // chunk of that stream as wave `wave` sees it.
+    struct Item {
+        int valid, c, r, b, h, tile, p0;           // r: position of the chunk in its work item
+        __amdgpu_buffer_rsrc_t rsx, rsB;
+        const float *dtp, *dap;
+        const int32_t *sqb;
+    };
+    // chunk r of the item behind ticket t (a ticket past the end, or a chunk past the sequence, gives an invalid
+    // chunk whose requests fetch nothing)
+    auto decode = [&](int t, int r) {
+        Item I;
+        const int tv = t < total ? t : 0;
+        const int k = tv / n_units;
+        I.c = k * R + r;
+        I.r = r;
+        I.valid = t < total && I.c < C;
+        if (!I.valid) I.c = 0;
+        I.tile = 4 * (unit0 + tv - k * n_units) + wave;
+        const int r1 = I.tile / n_pt;
+        I.p0 = 32 * (I.tile - r1 * n_pt);
+        I.b = r1 / p.nheads;
+        I.h = r1 - I.b * p.nheads;
+        const int g = I.h / (p.nheads / p.ngroups);
+        // descriptor of the chunk: base = its first token, extent = the tokens that exist
+        const char *xb = (const char *)p.x + 2 * (I.b * p.sx_b + I.h * p.sx_h) + (int64_t)I.c * Q * xrb;
+        const char *Bb = (const char *)p.B + 2 * (I.b * p.sB_b + g * p.sB_g) + (int64_t)I.c * Q * Brb;
+        I.rsx = make_rsrc(xb, I.valid ? (int64_t)(L - I.c * Q) * xrb : 0);
+        I.rsB = make_rsrc(Bb, I.valid ? (int64_t)(L - I.c * Q) * Brb : 0);
+        I.dtp = p.dt + I.b * p.sdt_b + I.h * p.sdt_h + (int64_t)I.c * p.sdt_c;
+        I.dap = p.dacs + I.b * p.sda_b + I.h * p.sda_h + (int64_t)I.c * p.sda_c;
+        I.sqb = HAS_SEQ ? p.seq + I.b * p.ssq_b : nullptr;
+        return I;
+    };
+    // the chunk after I in the stream: the item's next chunk, or the first chunk of the item behind ticket t_next
+    auto successor = [&](const Item &I, int t_cur, int t_next) {
+        if (I.r + 1 < R && I.c + 1 < C) {
+            Item J = I;             // same tile, one chunk on
+            (void)t_cur;
+            J.c = I.c + 1;
+            J.r = I.r + 1;
+            const int g = I.h / (p.nheads / p.ngroups);
+            const char *xb = (const char *)p.x + 2 * (I.b * p.sx_b + I.h * p.sx_h) + (int64_t)J.c * Q * xrb;
+            const char *Bb = (const char *)p.B + 2 * (I.b * p.sB_b + g * p.sB_g) + (int64_t)J.c * Q * Brb;
+            J.rsx = make_rsrc(xb, (int64_t)(L - J.c * Q) * xrb);
+            J.rsB = make_rsrc(Bb, (int64_t)(L - J.c * Q) * Brb);
+            J.dtp = I.dtp + p.sdt_c;
+            J.dap = I.dap + p.sda_c;
+            return J;
+        }
+        return decode(t_next, 0);
+    };
+
+    // ---- request helpers (layouts as in ssd_quad.hip) ---------------------------------------------------------
+    // A step's B tile (32 tokens x dstate) sits in LDS as NT blocks of 1 KB, block (th, pair) = 16 tokens (token
+    // half th) x 32 columns (column pair `pair`), row-major: one request fetches a block, lane l the 16 bytes
+    // (token l/4, piece l%4) and deposits them at byte 16*l.  For the tokens 8..15 of a block the two 32-byte halves
+    // are swapped (piece ^ 2), which keeps the transposing reads below off shared banks.
+    const int Blane = (int)((lane >> 2) * Brb) + 16 * ((lane & 3) ^ ((lane >> 5) << 1));
+    auto load_B = [&](__amdgpu_buffer_rsrc_t rs, int s, int bi) {       // block bi of step s of the chunk behind rs
+#if defined(__HIP_DEVICE_COMPILE__)      // the LDS address space does not exist in the host pass
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+        const int th = bi / (NT / 2), pair = bi % (NT / 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRing) * NT + bi) * 1024), 16, Blane,
+                                                 (int)((32 * s + 16 * th) * Brb) + 64 * pair, 0, 0);
+#else
+        (void)rs; (void)s; (void)bi; (void)Blane;
+#endif
+    };
+    // The transposing read for (16 columns `it`, tokens 8kg + 4*half .. +3): lane (i16, kg) addresses the 8 bytes of
+    // token 8kg + 4*half + i16/4, columns 4*(i16%4)..+3 of that column block and receives column i16 of those four
+    // tokens.  Inline assembly with explicit s_waitcnt: given the intrinsic, the compiler would order every such
+    // read behind ALL outstanding loads that write LDS.
+    uint32_t Btr[2];
+    Btr[0] = (kg >> 1) * (NT / 2) * 1024 + (8 * (kg & 1) + (i16 >> 2)) * 64 + (kg & 1) * 32 + (i16 & 3) * 8;   // + 256 * half
+    Btr[1] = Btr[0] ^ 32;
+#if defined(__HIP_DEVICE_COMPILE__)
+    Btr[0] += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
+    Btr[1] += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)bring;
+#endif
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wunused-lambda-capture"   // the host pass sees no use of Btr
+    const uint32_t Btr0 = Btr[0], Btr1 = Btr[1];
+    auto read_Bt = [&, Btr0, Btr1](auto slotc, auto itc, u32x2 &lo, u32x2 &hi) {    // ring slot, column block
+        constexpr int it = decltype(itc)::value;
+        constexpr int off = (decltype(slotc)::value * NT + (it >> 1)) * 1024;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                     : "=&v"(lo), "=&v"(hi) : "v"((it & 1) ? Btr1 : Btr0), "n"(off), "n"(off + 256) : "memory");
+#else
+        lo = hi = (u32x2){0u, 0u}; (void)Btr0; (void)Btr1; (void)off;
+#endif
+    };
+#pragma clang diagnostic pop
+    // The results of a read_Bt become valid here: LDS operations complete in order, so the pair has arrived once no
+    // more LDS operations are outstanding than were issued after it (nc = that number, at least).
+    auto wait_Bt = [&](auto nc, u32x2 &lo, u32x2 &hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(decltype(nc)::value) : "memory");
+#else
+        (void)lo; (void)hi;
+#endif
+    };
+    // x: two requests cover the 32 token rows of a step, 4 lanes per 64-byte row of the slice; lane l deposits its
+    // 16 bytes at byte 16*l of a 1 KB block.  Request i fetches tokens 8*kg' + 4*i + m into row slot 4*m + kg'
+    // (kg' = (l/4)%4, m = l/16), so the four kg groups of an operand read below hit different banks.
+    const int xlane0 = (int)((8 * ((lane >> 2) & 3) + (lane >> 4)) * xrb) + 16 * (lane & 3);
+    auto load_x = [&](__amdgpu_buffer_rsrc_t rs, int p0, int s, int i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(xring + (s % kRing) * 2048 + i * 1024), 16, xlane0 + 2 * p0,
+                                                 (int)((32 * s + 4 * i) * xrb), 0, 0);
+#else
+        (void)rs; (void)p0; (void)s; (void)i; (void)xlane0;
+#endif
+    };
+    const int xst_rd = 64 * kg + 4 * i16;     // + 2048 * slot + 1024 * (j/4) + 256 * (j%4) for token 8kg + j
+
+    // decay inputs of an item's chunk: TPL consecutive tokens per lane, plus the chunk-level scalars
+    struct Meta { float dtv[TPL], cs[TPL], last; int32_t id[TPL], id_last, id_prev; };
+    auto load_meta = [&](const Item &I) {
+        Meta m;
+        const float *dtp = I.dtp + TPL * lane;
+        const float *dap = I.dap + TPL * lane;
+        if constexpr (TPL == 4) {
+            const f32x4 a = *(const f32x4 *)dtp, d = *(const f32x4 *)dap;
+            m.dtv[0] = a.x; m.dtv[1] = a.y; m.dtv[2] = a.z; m.dtv[3] = a.w;
+            m.cs[0] = d.x; m.cs[1] = d.y; m.cs[2] = d.z; m.cs[3] = d.w;
+        } else {
+            const f32x2 a = *(const f32x2 *)dtp, d = *(const f32x2 *)dap;
+            m.dtv[0] = a.x; m.dtv[1] = a.y; m.cs[0] = d.x; m.cs[1] = d.y;
+        }
+        m.last = I.dap[Q - 1];
+        m.id_last = m.id_prev = 0;
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) m.id[t] = 0;
+        if (HAS_SEQ) {
+#pragma unroll
+            for (int t = 0; t < TPL; ++t) m.id[t] = I.sqb[(int64_t)min(I.c * Q + TPL * lane + t, L - 1) * p.ssq_l];
+            m.id_last = I.sqb[(int64_t)(min((I.c + 1) * Q, L) - 1) * p.ssq_l];
+            // id of the previous chunk's last token; the recurrence starts from id 0 (kernels/ssd_state_passing.py:68)
+            if (I.c > 0) m.id_prev = I.sqb[(int64_t)(I.c * Q - 1) * p.ssq_l];
+        }
+        return m;
+    };
+    // per-token weights of a chunk (kernels/ssd_chunk_state.py:134-156) -> weight slot ws
+    auto put_weights = [&](int c, int ws, const Meta &m) {
+        float w[TPL];
+#pragma unroll
+        for (int t = 0; t < TPL; ++t) {
+            float e = m.last - m.cs[t];
+            if (p.clamp) e = fminf(e, 0.f);
+            w[t] = __expf(e) * m.dtv[t];
+            if (c * Q + TPL * lane + t >= L) w[t] = 0.f;
+            if (HAS_SEQ && m.id[t] != m.id_last) w[t] = 0.f;
+        }
+        if constexpr (TPL == 4) *(f32x4 *)(wbuf + ws * Q * 4 + 16 * lane) = (f32x4){w[0], w[1], w[2], w[3]};
+        else *(f32x2 *)(wbuf + ws * Q * 4 + 8 * lane) = (f32x2){w[0], w[1]};
+    };
+
+    // ---- operand helpers -------------------------------------------------------------------------------------
+    // x dwords (token, headdim row pair i16) and weights of the 8 tokens 8kg..8kg+7 of step s
+    auto read_operands = [&](int s, int ws, uint32_t (&xr)[8], float (&wv)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            xr[j] = *(const uint32_t *)(xring + (s % kRing) * 2048 + xst_rd + 1024 * (j >> 2) + 256 * (j & 3));
+        const f32x4 wlo = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg));
+        const f32x4 whi = *(const f32x4 *)(wbuf + ws * Q * 4 + 4 * (32 * s + 8 * kg + 4));
+        wv[0] = wlo.x; wv[1] = wlo.y; wv[2] = wlo.z; wv[3] = wlo.w;
+        wv[4] = whi.x; wv[5] = whi.y; wv[6] = whi.z; wv[7] = whi.w;
+    };
+    // tokens (2q, 2q+1) of headdim row 2*i16 + jp: x * w in fp32, split into bf16 hi + bf16 lo
+    auto frag_piece = [&](int q, int jp, const uint32_t (&xr)[8], const float (&wv)[8], Frag &f) {
+        const uint32_t r0 = xr[2 * q], r1_ = xr[2 * q + 1];
+        const float x0 = __builtin_bit_cast(float, jp ? (r0 & 0xffff0000u) : (r0 << 16));
+        const float x1 = __builtin_bit_cast(float, jp ? (r1_ & 0xffff0000u) : (r1_ << 16));
+        uint32_t hp = pack_bf16(x0 * wv[2 * q], x1 * wv[2 * q + 1]);
+        asm volatile("" : "+v"(hp));      // keeps the compiler from converting the product a second time to get h0
+        const float h0 = __builtin_bit_cast(float, hp << 16);
+        const float h1 = __builtin_bit_cast(float, hp & 0xffff0000u);
+        f.hi[jp][q] = hp;
+        // the residual of the exact product, as a fused multiply-add everywhere
+        f.lo[jp][q] = pack_bf16(__builtin_fmaf(x0, wv[2 * q], -h0), __builtin_fmaf(x1, wv[2 * q + 1], -h1));
+    };
+
+    // acc[it][jp][r]: dstate column 16*it + 4*kg + r of headdim row p0 + 2*i16 + jp
+    f32x4 acc[NT][2];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int it = 0; it < NT; ++it)
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp) acc[it][jp] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    };
+
+    // ---- chunk states parked in registers, and the chain step of an item --------------------------------------
+    // The accumulators hold a 16 x 16 block as (lane%16 = row, lane/16 = group of four columns); each block passes
+    // through 1 KB of LDS and comes back as (lane/4 = row, lane%4 = group), so that four adjacent lanes read and
+    // write 64 contiguous bytes of a state row (the memory pipeline merges only what adjacent lanes address).  The
+    // column group is XORed with row/4 in LDS, which keeps both the 16-byte writes and reads off shared banks.  A
+    // chunk state is parked in that layout: held[r][j] = block j of chunk r of the item, scale[r] its decay.
+    f32x4 held[R][2 * NT];
+    float scale[R];
+    auto park_into = [&](f32x4 (&dst)[2 * NT]) {
+        f32x4 *wr = (f32x4 *)(stage + i16 * 64 + ((kg ^ (i16 >> 2)) << 4));
+        const f32x4 *rd = (const f32x4 *)(stage + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4));
+        // LDS operations of one wave execute in order, so block k + 1 may be written right behind the read of block k
+#pragma unroll
+        for (int k = 0; k < 2 * NT; ++k) {
+            *wr = acc[k >> 1][k & 1];
+            dst[k] = *rd;
+        }
+    };
+    auto park = [&](const Item &I, const Meta &m) {
+        float sc = __expf(m.last);
+        if (HAS_SEQ && m.id_last != m.id_prev) sc = 0.f;
+        sc = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, sc)));
+        static_for<R>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            if (I.r == r) { park_into(held[r]); scale[r] = sc; }
+        });
+    };
+    // A flag poll must not be served by the per-CU cache: a device-scope load (sc1) misses there (sc0 does not:
+    // measured) and is answered by the L2, where a LOCAL producer's plain store has put the flag, or by memory, where
+    // a GLOBAL producer's device-scope store has.
+    auto load_flag = [&](const int *f) { return __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    auto raise_flag = [&](int *f) {
+        if (lane == 0) {
+            if (LOCAL) *(volatile int *)f = 1;
+            else __hip_atomic_store(f, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+    // I: the last chunk of the item (chunks I.c - I.r .. I.c)
+    auto chain_step = [&](const Item &I) {
+        const int c0 = I.c - I.r, n = I.r + 1;
+        const bool use_prev = (c0 > 0 || p.init != nullptr) && scale[0] != 0.f;
+        const int64_t slice_out = (int64_t)(p.headdim - 1) * p.so_p + p.dstate;
+        const int64_t slice_fin = (int64_t)(p.headdim - 1) * p.sf_p + p.dstate;
+        const int64_t slice_in = (int64_t)(p.headdim - 1) * p.sin_p + p.dstate;
+        const float *outb = (const float *)p.out + I.b * p.so_b + I.h * p.so_h;
+        const __amdgpu_buffer_rsrc_t rs_prev =
+            c0 > 0 ? make_rsrc(outb + (int64_t)c0 * p.so_c, slice_out * 4)
+                   : make_rsrc((const float *)p.init + I.b * p.sin_b + I.h * p.sin_h, p.init ? slice_in * 4 : 0);
+        const int pitch_prev = c0 > 0 ? (int)p.so_p : (int)p.sin_p;
+        const int row = I.p0 + 2 * (lane >> 2), col = 4 * (lane & 3);
+        int *const flag = ws_flags + (int64_t)I.tile * C;
+        // chunk j of the item ends in out[:, c0 + j + 1], the sequence's last chunk in final_states
+        auto store_chunk = [&](int j, const f32x4 (&v)[2 * NT], int aux) {
+            const bool fin = c0 + j + 1 == C;
+            const __amdgpu_buffer_rsrc_t rs = fin ? make_rsrc(p.fin + I.b * p.sf_b + I.h * p.sf_h, slice_fin * 4)
+                                                  : make_rsrc(outb + (int64_t)(c0 + j + 1) * p.so_c, slice_out * 4);
+            const int pitch = fin ? (int)p.sf_p : (int)p.so_p;
+#pragma unroll
+            for (int k = 0; k < 2 * NT; ++k) store4_f32(rs, row * pitch + col, (k & 1) * pitch + 16 * (k >> 1), v[k], aux);
+        };
+
+        if (use_prev && c0 > 0) {
+            // out[:, c0] of this tile is complete once its flag is up
+            int polls = 0;
+            while (load_flag(flag + c0) == 0) {
+                __builtin_amdgcn_s_sleep(1);
+                if (++polls >= p.spin_limit) {
+                    if (lane == 0) __hip_atomic_fetch_or(ws_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+            }
+            asm volatile("" ::: "memory");
+        }
+        if (use_prev || c0 == 0) {
+            f32x4 s[2 * NT];
+            const bool read = use_prev || p.init != nullptr;        // chunk 0 copies initial_states to out[:, 0] even
+#pragma unroll                                                      // if a sequence boundary wipes them out at once
+            for (int k = 0; k < 2 * NT; ++k) {
+                s[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                if (read)
+                    s[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                         rs_prev, 4 * (row * pitch_prev + col),
+                                                         4 * ((k & 1) * pitch_prev + 16 * (k >> 1)), kAux));
+            }
+            if (use_prev) {
+                // the recurrence over the item's chunks, in place: held[j] becomes the state after chunk c0 + j
+                static_for<R>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    if (j < n) {
+                        const float sc = scale[j];
+#pragma unroll
+                        for (int k = 0; k < 2 * NT; ++k) {
+                            const f32x4 pv = j == 0 ? s[k] : held[j > 0 ? j - 1 : 0][k];
+                            held[j][k] = (f32x4){__builtin_fmaf(pv.x, sc, held[j][k].x), __builtin_fmaf(pv.y, sc, held[j][k].y),
+                                                 __builtin_fmaf(pv.z, sc, held[j][k].z), __builtin_fmaf(pv.w, sc, held[j][k].w)};
+                        }
+                    }
+                });
+            }
+            if (c0 == 0) {
+#pragma unroll
+                for (int k = 0; k < 2 * NT; ++k)
+                    store4_f32(make_rsrc(outb, slice_out * 4), row * (int)p.so_p + col, (k & 1) * (int)p.so_p + 16 * (k >> 1), s[k], 0);
+            }
+        }
+        if (!use_prev) {
+            // the item starts a sequence: its first state is its first chunk state
+            static_for<R>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if (j >= 1 && j < n) {
+                    const float sc = scale[j];
+#pragma unroll
+                    for (int k = 0; k < 2 * NT; ++k) {
+                        const f32x4 pv = held[j > 0 ? j - 1 : 0][k];
+                        held[j][k] = (f32x4){__builtin_fmaf(pv.x, sc, held[j][k].x), __builtin_fmaf(pv.y, sc, held[j][k].y),
+                                             __builtin_fmaf(pv.z, sc, held[j][k].z), __builtin_fmaf(pv.w, sc, held[j][k].w)};
+                    }
+                }
+            });
+        }
+        // the state the next item waits for first ...
+        static_for<R>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            if (j == n - 1) store_chunk(j, held[j], kAux);
+        });
+        if (c0 + n < C) {
+            // ... its stores have been acknowledged (by the L2 both sides share, or by memory) before the flag is raised.
+            // (Letting the next chunk's first wait for its own x rows stand in for this one -- memory operations
+            // complete in order -- saves the wait but raises the flag later: no gain at b=4 L=8192 H=80, and slower
+            // where the chain sets the pace: 1.19 ms instead of 1.10 ms at L=131072 H=128.)
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            asm volatile("" ::: "memory");
+            raise_flag(flag + c0 + n);
+        }
+        // ... then the states inside the item, which nobody waits for.  (Spreading these stores over the steps of the
+        // next item was measured: 250 us instead of 215 at b=4 L=8192 H=80 -- memory operations complete in order, so
+        // every later wait for a load also waits for the stores issued before it, and a store is acknowledged late.)
+        static_for<R>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            if (j < n - 1) store_chunk(j, held[j], 0);
+        });
+    };
+
+    // ---- tickets ---------------------------------------------------------------------------------------------
+    if (threadIdx.x == 0) {
+        const int t = __hip_atomic_fetch_add(ws_ticket, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tq[0] = t;
+        tq[1] = t + 1;
+    }
+    // rows past the end of the sequence are not fetched and leave their LDS slots untouched; their weight is zero,
+    // so the slots only have to hold finite numbers
+#pragma unroll
+    for (int i = 0; i < 2 * kRing; ++i) *(u32x4 *)(xring + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < kRing * NTW; ++i)
+        *(u32x4 *)(bring + (i * 4 + wave) * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
+    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): the zeros are in place before any row lands
+    __builtin_amdgcn_s_barrier();
+    // the tickets of the current and of the next item; the one after that is drawn while the current item runs
+    int t_cur = __builtin_amdgcn_readfirstlane(tq[0]), t_nxt = __builtin_amdgcn_readfirstlane(tq[1]);
+    Item cur = decode(t_cur, 0);
+    Item nxt = successor(cur, t_cur, t_nxt);
+    if (!cur.valid) return;                      // whole workgroup: no barrier is skipped
+
+    Meta mcur = load_meta(cur);
+    // requests of the steps 0..kDist-1, in the order (x, x, B...) that every later step keeps
+#pragma unroll
+    for (int s = 0; s < kDist; ++s) {
+        load_x(cur.rsx, cur.p0, s, 0); load_x(cur.rsx, cur.p0, s, 1);
+#pragma unroll
+        for (int k = 0; k < NTW; ++k) load_B(cur.rsB, s, wave * NTW + k);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    put_weights(cur.c, 0, mcur);
+    Frag fA, fB;
+    // B operands (transposed blocks) travel kAhead iterations ahead of the MFMAs that use them, across step and item
+    // boundaries: block t of the stream of (step, tile) pairs sits in slot t % 4
+    constexpr int kAhead = 3;
+    static_assert(NT % 4 == 0 && kAhead < 4 && kAhead <= NT, "slot of a block = its tile index % 4");
+    static_assert(SPC % kRing == 0, "ring slots repeat from item to item");
+    u32x2 blo[4], bhi[4];
+    {
+        // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 1) * (2 + NTW)));
+        __builtin_amdgcn_s_barrier();   // ... and every other wave's blocks of step 0
+        asm volatile("" ::: "memory");
+        uint32_t xr[8]; float wv[8];
+        read_operands(0, 0, xr, wv);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { frag_piece(q, 0, xr, wv, fA); frag_piece(q, 1, xr, wv, fA); }
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<kAhead>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            read_Bt(std::integral_constant<int, 0>{}, ic, blo[i], bhi[i]);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    Meta mnext = mcur;
+    int t_new = 0;          // the ticket drawn during this item (wave 0, lane 0)
+    zero_acc();
+    // One 32-token step s of the current item (weight slot ws): fc = x operands of this step, fn receives those of
+    // the step after it (the next item's first step after the last one).  Vector-memory requests of a step, in
+    // program order: the two x requests of step + 3 (iteration 0), this wave's B requests of step + 3 (after the
+    // barrier in iteration NT - kAhead); steps past the item's last belong to the next item.  Memory operations
+    // complete in order and the compiler does not track loads that write LDS, so the waits for them are explicit:
+    // "no more outstanding than were issued after the one needed".  Operations the counts leave out (the ticket
+    // draw, the next item's decay inputs) only make a wait longer than needed, never shorter; the chain step
+    // between two items ends with every operation complete.
+    auto step = [&](auto sc, int ws, Frag &fc, Frag &fn) {
+        constexpr int s = decltype(sc)::value;
+        // x rows of step + 1 (this wave's own, requested two steps ago): behind them came the B requests of that
+        // step and all requests of the steps s + 2 - kDist .. s - 1
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(NTW + (kDist - 2) * (2 + NTW)));
+        asm volatile("" ::: "memory");
+        uint32_t xr[8]; float wv[8];
+        if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
+        else read_operands(0, ws ^ 1, xr, wv);
+        if (s == 0 && cur.r == 0 && threadIdx.x == 0)
+            t_new = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (s == SPC - 2 && cur.r == 0 && threadIdx.x == 0) tq[2] = t_new;     // published by this step's barrier
+        // requests of this step: x rows and this wave's B blocks of step + 3 (this item or the next)
+        const auto rsB = s + kDist < SPC ? cur.rsB : nxt.rsB;
+        const auto rsx = s + kDist < SPC ? cur.rsx : nxt.rsx;
+        const int xp0 = s + kDist < SPC ? cur.p0 : nxt.p0;
+        const int s3 = (s + kDist) % SPC;
+        const bf16x8 h0 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[0][0], fc.hi[0][1], fc.hi[0][2], fc.hi[0][3]});
+        const bf16x8 h1 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[1][0], fc.hi[1][1], fc.hi[1][2], fc.hi[1][3]});
+        const bf16x8 l0 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[0][0], fc.lo[0][1], fc.lo[0][2], fc.lo[0][3]});
+        const bf16x8 l1 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[1][0], fc.lo[1][1], fc.lo[1][2], fc.lo[1][3]});
+        __builtin_amdgcn_sched_barrier(0);   // operand reads above, the requests of this step below
+        static_for<NT>([&](auto itc) {
+            constexpr int it = decltype(itc)::value;
+            // the kAhead - 1 blocks behind this one (two reads each) may still be in flight
+            wait_Bt(std::integral_constant<int, 2 * (kAhead - 1)>{}, blo[it % 4], bhi[it % 4]);
+            const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it % 4].x, blo[it % 4].y, bhi[it % 4].x, bhi[it % 4].y});
+            if constexpr (it == NT - kAhead) {
+                // The next read is the first of step + 1's tile: this wave's blocks of it (requested three steps
+                // ago) have landed once only the requests of step - 1 and the x requests of this step are
+                // outstanding; the barrier publishes every wave's blocks.  It also tells that all waves are through
+                // with the tile of step - 1, whose ring slot the B requests below overwrite.
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 2) * (2 + NTW) + 2));
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+            {
+                constexpr int tn = it + kAhead;     // block kAhead iterations on: this step's tile or the next one's
+                read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
+                        blo[tn % 4], bhi[tn % 4]);
+            }
+            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
+            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
+            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
+            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l1, acc[it][1], 0, 0, 0);
+            // next step's x operands, one or two eighths per iteration
+#pragma unroll
+            for (int e = it * 8 / NT; e < (it + 1) * 8 / NT; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
+            if (it == 0) { load_x(rsx, xp0, s3, 0); load_x(rsx, xp0, s3, 1); }
+            if (it >= NT - kAhead && it < NT - kAhead + NTW) load_B(rsB, s3, wave * NTW + (it - (NT - kAhead)));
+            if (s == 1 && it == NT - 1 && nxt.valid) mnext = load_meta(nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (s == SPC / 2) put_weights(nxt.c, ws ^ 1, mnext);
+    };
+
+    for (int n = 0; cur.valid; ++n) {
+        const int ws = n & 1;
+        step(std::integral_constant<int, 0>{}, ws, fA, fB);
+        step(std::integral_constant<int, 1>{}, ws, fB, fA);
+        step(std::integral_constant<int, 2>{}, ws, fA, fB);
+        step(std::integral_constant<int, 3>{}, ws, fB, fA);
+        if constexpr (SPC == 8) {
+            step(std::integral_constant<int, 4>{}, ws, fA, fB);
+            step(std::integral_constant<int, 5>{}, ws, fB, fA);
+            step(std::integral_constant<int, 6>{}, ws, fA, fB);
+            step(std::integral_constant<int, 7>{}, ws, fB, fA);
+        }
+        park(cur, mcur);
+        zero_acc();
+        if (!(cur.r + 1 < R && cur.c + 1 < C)) {
+            // the item's last chunk: the chain step, then the tickets move up
+            chain_step(cur);
+            t_cur = t_nxt;
+            t_nxt = __builtin_amdgcn_readfirstlane(tq[2]);
+        }
+        mcur = mnext;
+        cur = nxt;
+        nxt = successor(cur, t_cur, t_nxt);
+    }
+    if (LOCAL && threadIdx.x == 0) {
+        // every workgroup that drew from a slot's counter must sit on the same XCD; anything else (hardware ids that
+        // do not spread over p.n_xcd slots) would break the L2 argument above, and is reported instead of ignored
+        const int seen = __hip_atomic_fetch_max(p.ws + kWsOwner + slot, xcd_hw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (seen != 0 && seen != xcd_hw + 1) __hip_atomic_fetch_or(ws_err, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// workspace cleared before every launch: ticket counter, error word and flags
+__global__ void __launch_bounds__(256) clear_kernel(int *ws, int n)
+{
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = 0;
+}
+
+static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
+
+static bool rows_ok(const void *ptr, int64_t strides_or, int64_t row_stride, int headdim)
+{
+    return aligned(ptr, 16) && strides_or % 4 == 0 && (int64_t)headdim * row_stride < (1LL << 28);
+}
+
+}  // namespace chain
+
+size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks)
+{
+    const int64_t tiles = (int64_t)batch * nheads * ((headdim + 31) / 32);
+    return (size_t)(chain::kWsHeaderInts + tiles * nchunks) * sizeof(int);
+}
+
+// fp32 out / initial_states / final_states, no `states` output, and what the four-tile kernel asks of the inputs
+bool chain_supported(const Params &p)
+{
+    using namespace chain;
+    if (p.states || !p.out || !p.fin) return false;
+    if (!quad_inputs_supported(p)) return false;
+    if (p.dt_out != DT_F32 || (p.init && p.dt_init != DT_F32)) return false;
+    if (!rows_ok(p.out, p.so_b | p.so_c | p.so_h | p.so_p, p.so_p, p.headdim)) return false;
+    if (!rows_ok(p.fin, p.sf_b | p.sf_h | p.sf_p, p.sf_p, p.headdim)) return false;
+    if (p.init && !rows_ok(p.init, p.sin_b | p.sin_h | p.sin_p, p.sin_p, p.headdim)) return false;
+    if ((int64_t)p.batch * p.nheads * (p.headdim / 32) * p.C >= (1LL << 30)) return false;     // flag index, tickets
+    return true;
+}
+
+template <int NT, int SPC, int R, bool SEQ, bool LOCAL>
+static hipError_t launch_chain_k(const Params &p, int n_wg, hipStream_t s)
+{
+    constexpr int lds = chain::lds_bytes<NT, SPC>();
+    static std::atomic<uint64_t> configured{0};
+    const hipError_t e = ensure_dynamic_lds((const void *)chain::chain_kernel<NT, SPC, R, SEQ, LOCAL>, lds, configured);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((chain::chain_kernel<NT, SPC, R, SEQ, LOCAL>), dim3(n_wg), dim3(256), lds, s, p);
+    return hipGetLastError();
+}
+
+template <int R, bool SEQ, bool LOCAL>
+static hipError_t launch_chain_r(const Params &p, int n_wg, hipStream_t s)
+{
+    const int nt = p.dstate / 16, spc = p.Q / 32;
+    if (nt == 8 && spc == 8) return launch_chain_k<8, 8, R, SEQ, LOCAL>(p, n_wg, s);
+    if (nt == 8 && spc == 4) return launch_chain_k<8, 4, R, SEQ, LOCAL>(p, n_wg, s);
+    if (nt == 4 && spc == 8) return launch_chain_k<4, 8, R, SEQ, LOCAL>(p, n_wg, s);
+    return launch_chain_k<4, 4, R, SEQ, LOCAL>(p, n_wg, s);
+}
+
+template <bool SEQ, bool LOCAL>
+static hipError_t launch_chain_t(const Params &p, int r, int n_wg, hipStream_t s)
+{
+    if (r >= 4) return launch_chain_r<4, SEQ, LOCAL>(p, n_wg, s);
+    if (r >= 2) return launch_chain_r<2, SEQ, LOCAL>(p, n_wg, s);
+    return launch_chain_r<1, SEQ, LOCAL>(p, n_wg, s);
+}
+
+// p.ws: at least chain_workspace_bytes(...) of device memory, 4-byte aligned; the launch clears what it uses.
+// n_cu: compute units of the device.  mode: 0 = choose, 1 = LOCAL, 2 = GLOBAL.
+hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
+{
+    Params p = p_in;
+    p.n_items = p.batch * p.nheads * (p.headdim / 32);
+    if (p.n_items <= 0 || p.C <= 0) return hipSuccess;
+    if (p.spin_limit <= 0) p.spin_limit = 1 << 22;
+    const int64_t n_ws = chain::kWsHeaderInts + (int64_t)p.n_items * p.C;
+    hipLaunchKernelGGL(chain::clear_kernel, dim3((unsigned)((n_ws + 255) / 256 < 1024 ? (n_ws + 255) / 256 : 1024)), dim3(256), 0, s,
+                       p.ws, (int)n_ws);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    // An XCD is 32 compute units on this part.  Units are dealt to the XCDs in contiguous ranges; LOCAL pays when
+    // the fullest XCD holds at most an eighth more than its fair share of them.
+    const int n_units = p.n_items >> 2;
+    p.n_xcd = n_cu >= 32 ? n_cu / 32 : 1;
+    if (p.n_xcd > chain::kMaxXcd) p.n_xcd = chain::kMaxXcd;
+    // LOCAL pays when an XCD has enough units of its own to keep its compute units on different chains (measured:
+    // 20 units per XCD 213 against 224 us; 5 per XCD 568 against 254 us) and the units spread evenly.
+    const int fullest = (n_units + p.n_xcd - 1) / p.n_xcd;
+    const bool local = mode == 1 || (mode == 0 && n_units >= 16 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
+    // Chunks per item: as many as leave every workgroup a few items (the parked chunk states fill the register file:
+    // one workgroup per compute unit).  p.n_seg > 0 forces a value.
+    int r = p.n_seg > 0 ? p.n_seg : 4;
+    while (r > 1 && p.n_seg <= 0 && (int64_t)n_units * ((p.C + r - 1) / r) < 3 * (int64_t)n_cu) r >>= 1;
+    const int64_t total = (int64_t)n_units * ((p.C + r - 1) / r);
+    const int n_wg = (int)(total < n_cu ? total : n_cu);
+    if (p.seq) return local ? launch_chain_t<true, true>(p, r, n_wg, s) : launch_chain_t<true, false>(p, r, n_wg, s);
+    return local ? launch_chain_t<false, true>(p, r, n_wg, s) : launch_chain_t<false, false>(p, r, n_wg, s);
+}
+
+}  // namespace ssd

@@ -551,13 +551,9 @@ template <int NK, int PB, int MB, bool PLAIN, bool S16 = false>
 static hipError_t launch_scan_k(const ScanParams &p, hipStream_t s)
 {
     constexpr int lds = scan::lds_bytes<NK, PB, S16>();
-    static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
-    if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_kernel<NK, PB, MB, PLAIN, S16>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    const hipError_t e = ensure_dynamic_lds((const void *)scan::scan_states_kernel<NK, PB, MB, PLAIN, S16>, lds, configured);
+    if (e != hipSuccess) return e;
     const int64_t items = (int64_t)p.batch * p.C * p.nheads * (p.headdim / (16 * PB));
     hipLaunchKernelGGL((scan::scan_states_kernel<NK, PB, MB, PLAIN, S16>), dim3((unsigned)items), dim3(256), lds, s, p);
     return hipGetLastError();
@@ -585,13 +581,9 @@ template <int NK, int MBT, bool PLAIN>
 static hipError_t launch_heads_k(const ScanParams &p, int hb, hipStream_t s)
 {
     constexpr int lds = scan::heads_lds<NK, MBT>();
-    static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
-    if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)scan::scan_states_heads_kernel<NK, MBT, PLAIN>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    const hipError_t e = ensure_dynamic_lds((const void *)scan::scan_states_heads_kernel<NK, MBT, PLAIN>, lds, configured);
+    if (e != hipSuccess) return e;
     const int64_t items = (int64_t)p.batch * p.C * (p.nheads / hb) * (p.headdim / 64);
     hipLaunchKernelGGL((scan::scan_states_heads_kernel<NK, MBT, PLAIN>), dim3((unsigned)items), dim3(256), lds, s, p, hb);
     return hipGetLastError();
@@ -603,18 +595,18 @@ static hipError_t launch_heads_q(const ScanParams &p, int hb, hipStream_t s)
     return p.dt_out == DT_F32 && !p.accumulate ? launch_heads_k<NK, MBT, true>(p, hb, s) : launch_heads_k<NK, MBT, false>(p, hb, s);
 }
 
-static int g_scan_kernel = 0;       // 0 = choose, 1 = one workgroup per head, 2 = runs of heads
+// 0 = choose, 1 = one workgroup per head, 2 = runs of heads (process-wide tuning hook, atomic)
+static std::atomic<int> g_scan_kernel_hook{0};
 
 int set_scan_kernel(int k)
 {
-    const int old = g_scan_kernel;
-    g_scan_kernel = k;
-    return old;
+    return g_scan_kernel_hook.exchange(k);
 }
 
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s)
 {
     if ((int64_t)p.batch * p.seqlen * p.nheads * p.headdim == 0) return hipSuccess;
+    const int g_scan_kernel = g_scan_kernel_hook.load(std::memory_order_relaxed);
     if (scan_states_mfma_supported(p) && p.dt_states == DT_F32 && g_scan_kernel != 1 && p.headdim % 64 == 0 && p.sda_k == 1 &&
         ((uintptr_t)p.dacs % 16) == 0 && (p.sda_b | p.sda_h | p.sda_c) % 4 == 0) {
         // runs of heads: the longest divisor of the heads per group up to 10 (enough workgroups to fill the chip

@@ -588,14 +588,11 @@ static hipError_t launch_one(const Params &p, dim3 grid, hipStream_t s)
                        (!p.init || p.dt_init == DT_F32);
     constexpr int lds = lds_bytes<NB, KS, WV, FUSED>();
     // more than 64 KB of LDS per workgroup has to be requested explicitly, once per kernel
-    static bool configured[2] = {false, false};
-    if (lds > 65536 && !configured[all32]) {
-        hipError_t e = all32 ? hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, true>,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds)
-                             : hipFuncSetAttribute((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, false>,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    static std::atomic<uint64_t> configured[2];
+    {
+        const hipError_t e = all32 ? ensure_dynamic_lds((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, true>, lds, configured[1])
+                                   : ensure_dynamic_lds((const void *)mfma_kernel<NB, KS, WV, SEQ, FUSED, false>, lds, configured[0]);
         if (e != hipSuccess) return e;
-        configured[all32] = true;
     }
     if (all32) hipLaunchKernelGGL((mfma_kernel<NB, KS, WV, SEQ, FUSED, true>), grid, dim3(64 * WV), lds, s, p);
     else hipLaunchKernelGGL((mfma_kernel<NB, KS, WV, SEQ, FUSED, false>), grid, dim3(64 * WV), lds, s, p);
@@ -612,8 +609,8 @@ static hipError_t launch_nb_ks(const Params &p, bool fused, hipStream_t s)
     return seq ? launch_one<NB, KS, WV, true, false>(p, grid, s) : launch_one<NB, KS, WV, false, false>(p, grid, s);
 }
 
-static int g_force_split = 0;       // 0 = choose from the problem size; 2 or 4 = forced
-int set_token_split(int wv) { const int old = g_force_split; g_force_split = wv; return old; }
+static std::atomic<int> g_force_split{0};       // 0 = choose from the problem size; 2 or 4 = forced (process-wide hook)
+int set_token_split(int wv) { return g_force_split.exchange(wv); }
 
 hipError_t launch_mfma(const Params &p_in, bool fused, hipStream_t s)
 {
@@ -627,7 +624,8 @@ hipError_t launch_mfma(const Params &p_in, bool fused, hipStream_t s)
     // a tile serially with the running state in registers; there four waves win (2-wave workgroups spill and a
     // tile's chunk takes twice as long), 285 vs 361 us at b=4 L=8192 H=80.
     int wv = (!fused && p.n_items > 512) ? 2 : 4;
-    if (g_force_split == 2 || g_force_split == 4) wv = g_force_split;
+    const int forced = g_force_split.load(std::memory_order_relaxed);
+    if (forced == 2 || forced == 4) wv = forced;
     const int nb = p.dstate / 16, q128 = p.Q / 128;     // chunk 128 or 256
     if (wv == 4) {
         if (nb == 8 && q128 == 2) return launch_nb_ks<8, 2, 4>(p, fused, s);

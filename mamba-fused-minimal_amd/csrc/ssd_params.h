@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <utility>
 
 namespace ssd {
@@ -34,6 +35,9 @@ struct Params {
     int clamp;
     int n_items;          // work items of the launch
     int n_seg;            // segments the chunks are split into (chunk-state launch of the four-tile kernel)
+    int *ws;              // ticket counter, error word and flags of the ticket / flag-chain kernel
+    int spin_limit;       // polls after which a wave of that kernel stops waiting for a flag
+    int n_xcd;            // XCDs (L2 caches) the units of that kernel are dealt to
 };
 
 // State passing on a flattened state axis.
@@ -128,6 +132,22 @@ __device__ __forceinline__ float wave_inclusive_sum(float x)
     return x;
 }
 
+// A launch that asks for more than 64 KB of LDS needs hipFuncAttributeMaxDynamicSharedMemorySize set on the kernel
+// first, once per device.  `done` (one per kernel instantiation) has a bit per device ordinal, set after the call
+// succeeded: threads that launch a kernel for the first time together set the attribute twice, which is harmless.
+inline hipError_t ensure_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done)
+{
+    if (bytes <= 65536) return hipSuccess;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = dev >= 0 && dev < 64 ? 1ull << dev : 0;
+    if (bit && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
+
 // Launchers implemented in the .hip files; each returns the hipError_t of its launch.
 hipError_t launch_mfma(const Params &p, bool fused, hipStream_t s);
 hipError_t launch_generic(const Params &p, bool fused, hipStream_t s);
@@ -135,12 +155,14 @@ hipError_t launch_state_passing(const PassParams &p, hipStream_t s);
 bool mfma_supported(const Params &p);
 hipError_t launch_quad(const Params &p, hipStream_t s);     // fused, four state tiles per workgroup sharing B in LDS
 bool quad_supported(const Params &p);
-hipError_t launch_step_split(const Params &p, hipStream_t s);   // fused: three tiles per workgroup, steps dealt to the waves
-bool step_split_supported(const Params &p);
 hipError_t launch_quad_chunk_state(const Params &p, hipStream_t s);     // chunk states only, same kernel
 bool quad_chunk_state_supported(const Params &p);
 bool quad_inputs_supported(const Params &p);     // what the four-tile kernel asks of x, B, dt, dA_cumsum and the shape
 int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup of the above; returns the old value
+// fused, work items drawn by ticket and chained by flags: every compute unit busy whatever the number of tiles
+hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
+bool chain_supported(const Params &p);
+size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

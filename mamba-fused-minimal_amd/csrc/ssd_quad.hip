@@ -600,13 +600,9 @@ template <int NT, int SPC, bool SEQ, bool F32IO, bool CO>
 static hipError_t launch_quad_k(const Params &p, dim3 grid, hipStream_t s)
 {
     constexpr int lds = quad::lds_bytes<NT, SPC>();
-    static bool configured = false;     // more than 64 KB of LDS has to be requested explicitly, once per kernel
-    if (lds > 65536 && !configured) {
-        hipError_t e = hipFuncSetAttribute((const void *)quad::quad_kernel<NT, SPC, SEQ, F32IO, CO>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    const hipError_t e = ensure_dynamic_lds((const void *)quad::quad_kernel<NT, SPC, SEQ, F32IO, CO>, lds, configured);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL((quad::quad_kernel<NT, SPC, SEQ, F32IO, CO>), grid, dim3(256), lds, s, p);
     return hipGetLastError();
 }
@@ -638,8 +634,9 @@ hipError_t launch_quad(const Params &p_in, hipStream_t s)
     return launch_quad_c<false>(p, s);
 }
 
-static int g_segment_chunks = 0;     // 0 = choose; otherwise the chunks a workgroup walks in the chunk-state launch
-int set_quad_segment_chunks(int n) { const int old = g_segment_chunks; g_segment_chunks = n; return old; }
+// 0 = choose; otherwise the chunks a workgroup walks in the chunk-state launch (process-wide tuning hook, atomic)
+static std::atomic<int> g_segment_chunks{0};
+int set_quad_segment_chunks(int n) { return g_segment_chunks.exchange(n); }
 
 hipError_t launch_quad_chunk_state(const Params &p_in, hipStream_t s)
 {
@@ -650,7 +647,7 @@ hipError_t launch_quad_chunk_state(const Params &p_in, hipStream_t s)
     // workgroup + 0.4): a workgroup's first requests have nothing to hide behind, which costs about 0.4 of a chunk,
     // and the compute unit with the most workgroups finishes last (b=4 L=8192 H=80: 190 / 162 / 160 / 177 / 219 us
     // for 1 / 2 / 4 / 8 / 32 chunks per workgroup).
-    int cps = g_segment_chunks;
+    int cps = g_segment_chunks.load(std::memory_order_relaxed);
     if (cps <= 0) {
         double best = 0;
         for (int k = 1; k <= p.C; ++k) {

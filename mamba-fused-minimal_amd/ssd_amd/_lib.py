@@ -13,7 +13,8 @@ SSD_F32, SSD_BF16, SSD_F16 = 0, 1, 2
 _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_F16}
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
-           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
+           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes",
+           "ssd_fused_workspace_status", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
 class SsdTensor(ctypes.Structure):
@@ -25,6 +26,14 @@ class SsdDims(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in
                 ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk_size", "nchunks")]
 
+
+class SsdFusedOpts(ctypes.Structure):
+    _fields_ = [("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64), ("spin_limit", ctypes.c_int32),
+                ("kernel", ctypes.c_int32), ("chunks_per_item", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
+SSD_KERNEL_AUTO, SSD_KERNEL_CHAIN, SSD_KERNEL_CHAIN_LOCAL, SSD_KERNEL_CHAIN_GLOBAL = 0, 1, 2, 3
+SSD_ERR_SCRATCH, SSD_ERR_CHAIN_TIMEOUT = -6, -7
 
 _lib = None
 
@@ -49,6 +58,12 @@ def load():
     lib.ssd_state_passing_fwd.argtypes = [T, T, T, T, T, T, i32, i32, i32, i32, i32, i32, vp]
     lib.ssd_fused_chunk_state_passing_fwd.restype = ctypes.c_int
     lib.ssd_fused_chunk_state_passing_fwd.argtypes = [T, T, T, T, T, T, T, T, T, D, ctypes.c_int, vp]
+    lib.ssd_fused_chunk_state_passing_fwd_ws.restype = ctypes.c_int
+    lib.ssd_fused_chunk_state_passing_fwd_ws.argtypes = [T, T, T, T, T, T, T, T, T, D, ctypes.c_int, ctypes.POINTER(SsdFusedOpts), vp]
+    lib.ssd_fused_workspace_bytes.restype = ctypes.c_uint64
+    lib.ssd_fused_workspace_bytes.argtypes = [D]
+    lib.ssd_fused_workspace_status.restype = ctypes.c_int
+    lib.ssd_fused_workspace_status.argtypes = [vp, vp]
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.restype = ctypes.c_int
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.argtypes = [T] * 11 + [D, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, vp]
     lib.ssd_query_path.restype = ctypes.c_int

@@ -36,7 +36,8 @@ def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
     return B, x, dt, dA_cumsum, seq_idx
 
 
-def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
+def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True, _clamp=True):
+    # _clamp=False evaluates the decay as the reference's fused kernels do (no min(., 0), fused_globalbar.py:106)
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = B.shape
@@ -58,7 +59,7 @@ def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_f
     with torch.cuda.device(x.device):
         rc = lib.ssd_chunk_state_fwd(_lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt),
                                      _lib.tensor_arg(dA_cumsum), _lib.tensor_arg(seq_idx), _lib.tensor_arg(states),
-                                     dims, 1, _stream(x))
+                                     dims, 1 if _clamp else 0, _stream(x))
     _lib.check(rc, "ssd_chunk_state_fwd")
     return states
 
@@ -98,11 +99,19 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
 
 
 def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=None, seq_idx=None,
-                                         states=None, states_in_fp32=True, _clamp=True):
+                                         states=None, states_in_fp32=True, _clamp=True, _kernel=0, _spin_limit=0,
+                                         _workspace=None, _chunks_per_item=0):
     """One launch for chunk state + state passing.  Returns (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32).
 
     Unlike the reference's fused wrappers, the per-chunk states are an internal quantity that never reaches
-    memory unless the caller passes a ``states=`` buffer, which is then filled as a side effect."""
+    memory unless the caller passes a ``states=`` buffer, which is then filled as a side effect.
+
+    The reference's wrappers allocate their counters per call (kernels/fused_globalbar.py:237-238,
+    kernels/fused_concurrent.py:296-298); so does this one: a small int32 workspace for the ticket counter and the
+    flags of the kernel that spreads a sequence's chunks over all compute units.  ``_kernel`` (0 = let the library
+    choose, 1 = insist on that kernel, 2 / 3 = and on its per-XCD / device-wide variant), ``_chunks_per_item``
+    (1, 2 or 4 consecutive chunks per work item of that kernel, 0 = choose), ``_spin_limit`` (polls before a flag wait gives up, 0 = default) and
+    ``_workspace`` (an int32 tensor to use instead of allocating one) are test and tuning hooks."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = B.shape
@@ -130,13 +139,25 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     if initial_states is not None and initial_states.stride(-1) != 1:
         initial_states = initial_states.contiguous()
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    if _workspace is None:
+        _workspace = torch.empty(((int(lib.ssd_fused_workspace_bytes(dims)) + 3) // 4,), device=x.device, dtype=torch.int32)
+    opts = _lib.SsdFusedOpts(_workspace.data_ptr(), _workspace.numel() * 4, int(_spin_limit), int(_kernel),
+                             int(_chunks_per_item), 0)
     with torch.cuda.device(x.device):
-        rc = lib.ssd_fused_chunk_state_passing_fwd(
+        rc = lib.ssd_fused_chunk_state_passing_fwd_ws(
             _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),
             _lib.tensor_arg(seq_idx), _lib.tensor_arg(initial_states), _lib.tensor_arg(states),
-            _lib.tensor_arg(out), _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, _stream(x))
-    _lib.check(rc, "ssd_fused_chunk_state_passing_fwd")
+            _lib.tensor_arg(out), _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, ctypes.byref(opts),
+            _stream(x))
+    _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states
+
+
+def _fused_workspace_status(workspace):
+    """Waits for the current stream and returns 0, or -7 if a flag wait of the last fused launch that used
+    ``workspace`` ran out (ssd_fused_workspace_status)."""
+    with torch.cuda.device(workspace.device):
+        return int(_lib.load().ssd_fused_workspace_status(ctypes.c_void_p(workspace.data_ptr()), _stream(workspace)))
 
 
 def _fused_chunk_state_state_passing_fwd_globalbar(B, x, dt, dA_cumsum, out_dtype, initial_states=None,

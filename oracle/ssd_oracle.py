@@ -26,8 +26,10 @@ token_scan_ref         no counterpart in the reference: token-serial y_t = C_t .
 token_recurrence_ref   no counterpart in the reference: an independent, chunk-free
                        evaluation of the same linear recurrence used to pin the two
                        chunked functions.
-make_inputs            kernels/rand_data.py:4-25 is the reference's only input recipe;
-                       the five benchmark configurations use their own seeded recipe.
+make_inputs            the five benchmark configurations' own seeded recipe.
+make_reference_inputs  kernels/rand_data.py:4-25, the reference's only input recipe (as main.py:166 draws it): the same
+                       shapes, element types and distributions from a CPU generator (the reference draws on the GPU,
+                       so the bits differ; the value ranges -- dt in [0.5, 1), A in (-1, 0], no softplus -- do not).
 
 Pin status: all functions pinned (see tests/test_oracle.py); none is "parity unpinned".
 """
@@ -406,6 +408,22 @@ def make_inputs(cfg_index, **override):
     C_ = dt.shape[2]
     res["dt_tok"] = dt.permute(0, 2, 3, 1).reshape(b, C_ * Q, H)[:, :L].contiguous()
     return res
+
+
+def make_reference_inputs(n_groups=1, dstate=128, nheads=80, headdim=64, seq_len=2048, dtype=torch.bfloat16,
+                          chunk_size=256, batch_size=1, seed=42):
+    """The reference's own test case (kernels/rand_data.py:4-25; main.py:166-179 runs it with dt_softplus=False,
+    dt_bias, no initial states, no seq_idx, out_dtype = C.dtype = bf16).  Returns x, A, B, C, D, dt, dt_bias in the
+    reference's order, on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((batch_size, seq_len, nheads, headdim), generator=g).to(dtype)
+    A = (torch.rand((nheads,), generator=g) * -1).to(dtype)                       # can be 0: no decay at all
+    B = torch.randn((batch_size, seq_len, n_groups, dstate), generator=g).to(dtype)
+    C = torch.randn((batch_size, seq_len, n_groups, dstate), generator=g).to(dtype)
+    D = torch.randn((nheads,), generator=g).to(dtype)
+    dt = (torch.rand((batch_size, seq_len, nheads), generator=g) * 0.5 + 0.5).to(dtype)
+    dt_bias = (torch.rand((nheads,), generator=g) * 0.5 - 0.25).to(dtype)
+    return x, A, B, C, D, dt, dt_bias
 
 
 def algorithmic_bytes(cfg, with_states=False):

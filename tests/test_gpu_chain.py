@@ -1,0 +1,164 @@
+"""GPU parity of the ticket / flag-chain kernel (ssd_fused_chunk_state_passing_fwd_ws), forced through the C ABI in
+each of its variants, against the CPU oracle on the same seeded inputs.
+
+The kernel replaces the reference's global barrier (kernels/fused_globalbar.py:130-137) and its completion counters
+and throttle semaphore (kernels/fused_concurrent.py:81-84, 141, 205-208); the reference has no test of either beyond
+main.py:164-190.  Tolerance: rtol 2e-3 / atol 1e-3 against the fp32 oracle (bf16 inputs, fp32 states)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-3, 1e-3
+LOCAL, GLOBAL = 2, 3            # SSD_KERNEL_CHAIN_LOCAL / SSD_KERNEL_CHAIN_GLOBAL
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import ssd_amd
+    from ssd_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return ssd_amd
+
+
+def _dev(t):
+    return None if t is None else t.cuda()
+
+
+def _mismatches(got, want, rtol=RTOL, atol=ATOL):
+    got, want = got.float().cpu(), want.float()
+    assert got.shape == want.shape
+    assert torch.isfinite(got).all()
+    err = (got - want).abs()
+    return int((err > atol + rtol * want.abs()).sum()), float(err.max())
+
+
+def _chain_case(ops, oracle, d, kernel, r, name, clamp=True, spin_limit=0):
+    x, B, dt, dAcs, seq, init = d["x"], d["B"], d["dt"], d["dA_cumsum"], d["seq_idx"], d["initial_states"]
+    want_out, want_fin = oracle.fused_ref(B, x, dt, dAcs, initial_states=init, seq_idx=seq, clamp=clamp)
+    ws = torch.full((max(1 << 16, 64 + x.shape[0] * x.shape[2] * (x.shape[3] // 32) * dt.shape[2]),), -1,
+                    dtype=torch.int32, device="cuda")           # garbage on purpose: the call clears what it uses
+    print(f"[{name}] kernel={kernel} chunks/item={r} x{tuple(x.shape)} seq={seq is not None} init={init is not None}", flush=True)
+    out, fin = ops._fused_chunk_state_state_passing_fwd(
+        _dev(B), _dev(x), _dev(dt), _dev(dAcs), torch.float32, initial_states=_dev(init), seq_idx=_dev(seq),
+        _clamp=clamp, _kernel=kernel, _chunks_per_item=r, _workspace=ws, _spin_limit=spin_limit)
+    status = ops._fused_workspace_status(ws)
+    assert status == 0, f"{name}: workspace status {status}"
+    for what, got, want in (("out", out, want_out), ("final", fin, want_fin)):
+        bad, worst = _mismatches(got, want)
+        print(f"[{name}.{what}] max_abs={worst:.3e} mismatches={bad}/{want.numel()}", flush=True)
+        assert bad == 0, f"{name}.{what}: {bad} mismatches, max abs err {worst:.3e}"
+    return out, fin
+
+
+SHAPES = [
+    dict(b=2, L=2048, H=8, init=True),                   # 8 chunks, initial states
+    dict(L=2000, H=8, nseq=5, init=True),                # ragged last chunk, packed sequences, initial states
+    dict(L=2304, H=8),                                   # 9 chunks: items of 2 or 4 chunks do not divide them
+    dict(Q=128, L=1408, N=64, H=8),                      # chunk 128 (four steps, ring of four), dstate 64
+    dict(P=128, H=4, G=2, L=1280),                       # headdim 128, grouped B
+    dict(P=96, H=4, L=1024),                             # three row slices per head: tiles of a unit straddle heads
+    dict(L=1, H=8),                                      # a single token
+    dict(L=257, H=8),                                    # one full chunk and one token
+    dict(b=1, L=8192, H=16, nseq=3),                     # 32 chunks on few units: every workgroup waits on the chain
+]
+
+
+@pytest.mark.parametrize("r", [1, 2, 4])
+@pytest.mark.parametrize("kernel", [LOCAL, GLOBAL], ids=["local", "global"])
+@pytest.mark.parametrize("kw", SHAPES, ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_chain_kernel_variants(ops, oracle, kw, kernel, r):
+    base = dict(b=2, L=1024, H=6, G=1)
+    base.update(kw)
+    _chain_case(ops, oracle, oracle.make_inputs(1, **base), kernel, r, f"chain.k{kernel}.r{r}")
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("cfg", [2, 3], ids=["cfg2", "cfg3"])
+def test_chain_kernel_at_benchmark_configs(ops, oracle, cfg):
+    # what the library picks for these two by itself (cfg 4 is compared slice-wise in test_gpu_parity.py)
+    d = oracle.make_inputs(cfg)
+    _chain_case(ops, oracle, d, 1, 0, f"chain.cfg{cfg}")
+
+
+def test_chain_matches_the_other_fused_kernels(ops, oracle):
+    # same inputs through the chain kernel and through the kernel the workspace-less entry point picks
+    d = oracle.make_inputs(2, b=2, L=4096, H=16)
+    out, fin = _chain_case(ops, oracle, d, LOCAL, 4, "chain.vs")
+    lib = __import__("ssd_amd")._lib
+    xd, Bd, dtd, dAd, initd = map(_dev, (d["x"], d["B"], d["dt"], d["dA_cumsum"], d["initial_states"]))
+    old = ops.set_token_split(1)       # keeps the library from picking the chain kernel
+    try:
+        out2, fin2 = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32, initial_states=initd)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_token_split(old)
+    assert float((out - out2).abs().max()) <= 1e-4 and float((fin - fin2).abs().max()) <= 1e-4
+    assert lib is not None
+
+
+def test_chain_without_the_clamp(ops, oracle):
+    # clamp = 0 is what the reference's fused kernels compute (fused_globalbar.py:106); it differs from the clamped
+    # form only where dA_cumsum is not monotone
+    d = oracle.make_inputs(1, b=2, L=2048, H=8)
+    g = torch.Generator().manual_seed(5)
+    d["dA_cumsum"] = d["dA_cumsum"] + 0.3 * torch.randn(d["dA_cumsum"].shape, generator=g)
+    a = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], clamp=True)[0]
+    b = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], clamp=False)[0]
+    assert float((a - b).abs().max()) > 1e-2            # the two semantics do differ on these inputs
+    for clamp in (True, False):
+        _chain_case(ops, oracle, d, LOCAL, 4, f"chain.clamp{int(clamp)}", clamp=clamp)
+
+
+def test_chain_bounded_wait_gives_up_and_reports(ops, oracle):
+    # Four units, 32 chunks each, one poll allowed: waves reach their chain step long before their predecessors
+    # have finished, give up, and say so.  The launch still drains (every wave raises its flag), and the next call
+    # on the same workspace is clean.
+    d = oracle.make_inputs(1, b=1, L=8192, H=8)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    ws = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+    ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=GLOBAL, _chunks_per_item=1, _workspace=ws,
+                                             _spin_limit=1)
+    assert ops._fused_workspace_status(ws) == -7        # SSD_ERR_CHAIN_TIMEOUT
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=GLOBAL, _chunks_per_item=1,
+                                                        _workspace=ws)
+    assert ops._fused_workspace_status(ws) == 0
+    assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+def test_chain_rejections(ops, oracle):
+    from ssd_amd import _lib
+    d = oracle.make_inputs(1, b=2, L=1024, H=8)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    small = torch.zeros(8, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="workspace"):                       # forced, workspace too small
+        ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=1, _workspace=small)
+    with pytest.raises(RuntimeError, match="workspace"):                       # forced, 16-bit out is not its job
+        ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, _kernel=1)
+    # left to itself the library falls back to its other kernels in both situations
+    out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _workspace=small)
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    torch.cuda.synchronize()
+    assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+    assert _lib.SSD_ERR_SCRATCH == -6
+
+
+def test_chain_back_to_back_and_other_stream(ops, oracle):
+    # the workspace is cleared by every call: launches back to back on one stream reuse it
+    d = oracle.make_inputs(2, b=1, L=4096, H=16)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    initd = _dev(d["initial_states"])
+    ws = torch.empty(1 << 16, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        results = [ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=initd, _kernel=LOCAL,
+                                                            _workspace=ws) for _ in range(4)]
+        assert ops._fused_workspace_status(ws) == 0
+    stream.synchronize()
+    for out, fin in results[1:]:
+        assert torch.equal(out, results[0][0]) and torch.equal(fin, results[0][1])
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    assert _mismatches(results[0][0], want_out)[0] == 0 and _mismatches(results[0][1], want_fin)[0] == 0
