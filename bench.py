@@ -5,7 +5,11 @@ One "step" = one fused launch over one batch of synthetic input (default workloa
 shape, b=4, L=8192, H=80, P=64, N=128, chunk 256, bf16 inputs, fp32 states, fp32 initial states).
 Prints ONE JSON line on stdout; details go to stderr.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu] [--no-per-config]
+
+Besides the headline workload the line carries `per_config`: the fused call timed the same way on each of the five
+benchmark configurations (microseconds, GB/s of algorithmic bytes, fraction of HBM peak, TFLOP/s, parity mismatches
+against the CPU oracle).
 """
 import argparse
 import json
@@ -18,11 +22,28 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E
-# HBM bytes per fused launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB -> bytes; the
-# factors are what the same counters read for a plain 1 GiB copy).  Keyed by workload name; see the rocprof summaries
-# kept with the repository.  None = not measured for that workload / kernel version.
-MEASURED_TRAFFIC_BYTES = {"cfg2_mamba2_2p7b": 730515354}
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+# HBM bytes per fused launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB -> bytes; the
+# factors are what the same counters read for a plain 1 GiB copy), keyed by workload name, together with the hash of
+# the kernel sources the measurement was made on (kernel_source_hash() below).  The counters cannot be read from
+# inside this script, so the figure is only reported while the sources still hash to the same value; otherwise
+# `roofline.traffic` is null.  The rocprof summaries are kept with the repository.
+MEASURED_TRAFFIC = {}
+KERNEL_SOURCES = ("ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_tile.h", "ssd_params.h", "ssd_capi.hip")
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "mamba-fused-minimal_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    m = MEASURED_TRAFFIC.get(workload)
+    return m["bytes"] if m and m["sources"] == kernel_source_hash() else None
 
 
 def log(*a):
@@ -37,11 +58,16 @@ def main():
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--sets", type=int, default=3, help="rotating input/output buffer sets (defeats cache reuse)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--no-per-config", action="store_true", help="skip the table over the five configurations")
+    ap.add_argument("--source-hash", action="store_true", help="print the hash of the kernel sources and exit")
     ap.add_argument("--with-states", action="store_true", help="also materialise the per-chunk states")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy three times (the known-size kernel that the FETCH_SIZE / "
                          "WRITE_SIZE counters are scaled by) and exit")
     args = ap.parse_args()
+    if args.source_hash:
+        print(kernel_source_hash())
+        return
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU only (the driver's boxes have one GPU, and the path needs "
               "no exchange across GPUs); run with --gpus 1", file=sys.stderr)
@@ -133,16 +159,30 @@ def main():
     _, scan_ev = timed(scan_states, max(5, args.steps // 4), 3)
     del prev_states, y_bufs
 
-    # parity of what was timed, on one batch row, against the CPU oracle
+    # parity of what was timed, over the whole batch, against the CPU oracle (the long grouped configuration on four
+    # heads of different groups: its fp32 oracle would not fit a few minutes)
+    def parity(idx, dd, out, fin):
+        if idx == 4:
+            ratio, bad, worst = dd["x"].shape[2] // dd["B"].shape[2], 0, 0.0
+            for h in (0, 17, 63, 127):
+                g = h // ratio
+                wo, wf = ssd_oracle.fused_ref(dd["B"][:, :, g:g + 1], dd["x"][:, :, h:h + 1], dd["dt"][:, h:h + 1], dd["dA_cumsum"][:, h:h + 1])
+                eo, ef = (out[:, :, h:h + 1].cpu() - wo).abs(), (fin[:, h:h + 1].cpu() - wf).abs()
+                bad += int((eo > 1e-3 + 2e-3 * wo.abs()).sum()) + int((ef > 1e-3 + 2e-3 * wf.abs()).sum())
+                worst = max(worst, float(eo.max()), float(ef.max()))
+            return bad, worst, "heads 0, 17, 63, 127"
+        wo, wf = ssd_oracle.fused_ref(dd["B"], dd["x"], dd["dt"], dd["dA_cumsum"], initial_states=dd["initial_states"], seq_idx=dd["seq_idx"])
+        eo, ef = (out.cpu() - wo).abs(), (fin.cpu() - wf).abs()
+        bad = int((eo > 1e-3 + 2e-3 * wo.abs()).sum()) + int((ef > 1e-3 + 2e-3 * wf.abs()).sum())
+        return bad, max(float(eo.max()), float(ef.max())), "whole batch"
+
     out, fin = fused(0)
     torch.cuda.synchronize()
+    bad, worst, scope = parity(args.config, d, out, fin)
+    log(f"[bench] parity ({scope}): max|err|={worst:.3e}, mismatches={bad}")
     sl = slice(0, 1)
     cut = lambda t: None if t is None else t[sl]
-    w_out, w_fin = ssd_oracle.fused_ref(d["B"][sl], d["x"][sl], d["dt"][sl], d["dA_cumsum"][sl],
-                                        initial_states=cut(d["initial_states"]), seq_idx=cut(d["seq_idx"]))
-    err = (out[sl].cpu() - w_out).abs()
-    bad = int((err > 1e-3 + 2e-3 * w_out.abs()).sum()) + int(((fin[sl].cpu() - w_fin).abs() > 1e-3 + 2e-3 * w_fin.abs()).sum())
-    log(f"[bench] parity (batch row 0): max|err|={float(err.max()):.3e}, mismatches={bad}")
+    del out, fin
 
     alg_bytes = ssd_oracle.algorithmic_bytes(cfg, with_states=args.with_states)
     alg_flops = ssd_oracle.algorithmic_flops(cfg)
@@ -166,7 +206,9 @@ def main():
                    "materialise_states": bool(args.with_states), "buffer_sets": nsets},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None if args.with_states else MEASURED_TRAFFIC_BYTES.get(cfg["name"]),
+                     "traffic": None if args.with_states else measured_traffic(cfg["name"]),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel sources with hash "
+                                       + kernel_source_hash() + " (null: not measured on these sources)",
                      "algorithmic_bytes": alg_bytes, "kernel_us": round(ev_step * 1e6, 2)},
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -176,7 +218,45 @@ def main():
         "chunk_scan_states_us": round(scan_ev * 1e6, 2),
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,
+        "parity_scope": scope,
     }
+
+    if not args.no_per_config:
+        # the same call, timed the same way, on each of the five configurations
+        table = {}
+        steps_pc = max(5, args.steps // 4)
+        for idx in range(5):
+            c = ssd_oracle.CONFIGS[idx]
+            if idx == args.config:
+                dd, ev = d, ev_step
+                o, f = fused(0)
+                torch.cuda.synchronize()
+                pbad, pworst, pscope = bad, worst, scope
+            else:
+                dd = ssd_oracle.make_inputs(idx)
+                n = 2 if idx == 4 else nsets
+                dev_sets = [{k: mv(dd[k]) for k in ("B", "x", "dt", "dA_cumsum", "initial_states", "seq_idx")}]
+                dev_sets += [{k: (None if v is None else v.clone()) for k, v in dev_sets[0].items()} for _ in range(n - 1)]
+
+                def call(i, dev_sets=dev_sets, n=n):
+                    s_ = dev_sets[i % n]
+                    return ssd_amd._fused_chunk_state_state_passing_fwd(
+                        s_["B"], s_["x"], s_["dt"], s_["dA_cumsum"], torch.float32, initial_states=s_["initial_states"],
+                        seq_idx=s_["seq_idx"])
+
+                _, ev = timed(call, steps_pc, 3)
+                o, f = call(0)
+                torch.cuda.synchronize()
+                pbad, pworst, pscope = parity(idx, dd, o, f)
+                del dev_sets
+            ab, af = ssd_oracle.algorithmic_bytes(c), ssd_oracle.algorithmic_flops(c)
+            table[f"cfg{idx}"] = {"workload": c["name"], "us": round(ev * 1e6, 2), "gbps": round(ab / ev / 1e9, 1),
+                                  "frac": round(ab / ev / 1e9 / HBM_PEAK_GBPS, 4), "tflops": round(af / ev / 1e12, 2),
+                                  "algorithmic_bytes": ab, "parity_mismatches": pbad, "parity_scope": pscope}
+            log(f"[bench] {c['name']}: {table[f'cfg{idx}']}")
+            del o, f, dd
+            torch.cuda.empty_cache()
+        res["per_config"] = table
 
     if not args.no_cpu:
         # reference math in fp32 PyTorch on this machine's host cores: one batch row of the workload

@@ -208,7 +208,9 @@ int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tens
  * intra-chunk half of the scan computed elsewhere) instead of overwriting it.  bf16 C with fp32 or bf16 states,
  * dstate 64/128, chunk size 64/128/256 and headdim % 32 == 0 run on the matrix cores: a fp32 state enters as bf16
  * hi + lo (the reference rounds the state to C's element type), a bf16 state as it is; everything else on a plain
- * FMA kernel.
+ * FMA kernel (one thread per output element, orders of magnitude slower).  Size limits of the matrix-core kernels: one
+ * chunk of C rows and one chunk of y rows (chunk_size * row pitch in bytes) must stay below 2 GiB; the sequence length
+ * itself is not limited by them.
  */
 int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states, const ssd_tensor *dA_cumsum,
                               const ssd_tensor *seq_idx, const ssd_tensor *y, const ssd_dims *dims, int accumulate,

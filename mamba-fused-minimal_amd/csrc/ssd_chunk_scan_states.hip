@@ -194,7 +194,11 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
         load_to_lds(rsS, sld + ins * 1024, row * (int)s_pitch + q * 16, 0);
     }
     const int64_t c_pitch = p.sC_l * 2;
-    const auto rsC = make_rsrc((const char *)p.Cm + 2 * (b * p.sC_b + g * p.sC_g), (int64_t)(p.seqlen - 1) * c_pitch + N * 2);
+    // descriptors start at the chunk's first token (byte offsets inside one are 32-bit: the limit is then a chunk's
+    // extent, not the sequence's) and end with the sequence
+    const int chunk_tokens = min(p.Q, p.seqlen - c * p.Q), wtok0 = wave * 16 * MB;
+    const auto rsC = make_rsrc((const char *)p.Cm + 2 * (b * p.sC_b + g * p.sC_g) + (int64_t)c * p.Q * c_pitch,
+                               (int64_t)(chunk_tokens - 1) * c_pitch + N * 2);
     // token (within the block) and global piece of this lane for load instruction i of a C block
     auto load_C = [&](int mb, int buf) {
 #pragma unroll
@@ -202,7 +206,7 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
             const int t = i * (64 / PRC) + lane / PRC;
             const int q = (lane % PRC) ^ (t & (PRC - 1));
             load_to_lds(rsC, cbuf + buf * 16 * N * 2 + i * 1024, t * (int)c_pitch + q * 16,
-                        (tok0 + 16 * mb) * (int)c_pitch);
+                        (wtok0 + 16 * mb) * (int)c_pitch);
         }
     };
     load_C(0, 0);
@@ -242,8 +246,8 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 
     const int64_t o_pitch = p.so_l;                 // elements
     const int esz = p.dt_out == DT_F32 ? 4 : 2;
-    const auto rsO = make_rsrc((char *)p.out + esz * (b * p.so_b + h * p.so_h + p0),
-                               ((int64_t)(p.seqlen - 1) * o_pitch + 16 * PB) * esz);
+    const auto rsO = make_rsrc((char *)p.out + esz * (b * p.so_b + h * p.so_h + p0 + (int64_t)c * p.Q * o_pitch),
+                               ((int64_t)(chunk_tokens - 1) * o_pitch + 16 * PB) * esz);
 
     // ---- 16-token blocks.  Vector-memory operations of this wave from here on, in program order per block:
     // the C requests of block mb + 2, then the block's PB stores (preceded by PB loads when accumulating; the
@@ -309,7 +313,7 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
 #pragma unroll
             for (int r = 0; r < PB / 2; ++r) {
                 const int t = r * (64 / OP2) + lane / OP2, pp = lane % OP2;
-                store_y8(rsO, p.dt_out, p.accumulate, t * (int)o_pitch + 8 * pp, (tok0 + 16 * mb) * (int)o_pitch, ya[r], yd[r]);
+                store_y8(rsO, p.dt_out, p.accumulate, t * (int)o_pitch + 8 * pp, (wtok0 + 16 * mb) * (int)o_pitch, ya[r], yd[r]);
             }
             continue;
         }
@@ -325,7 +329,7 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
             const int piece = lane % OP;
             f32x4 v = yv[r];
             const int voff = t * (int)o_pitch + 4 * piece;              // elements, from the block's first token
-            const int soff = (tok0 + 16 * mb) * (int)o_pitch;
+            const int soff = (wtok0 + 16 * mb) * (int)o_pitch;
             store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, soff, v);
         }
     }
@@ -404,13 +408,14 @@ __global__ void __launch_bounds__(256, 1) scan_states_heads_kernel(const ScanPar
     };
     {
         const int64_t c_pitch = p.sC_l * 2;
-        const auto rsC = make_rsrc((const char *)p.Cm + 2 * (b * p.sC_b + g * p.sC_g), (int64_t)(p.seqlen - 1) * c_pitch + N * 2);
+        const auto rsC = make_rsrc((const char *)p.Cm + 2 * (b * p.sC_b + g * p.sC_g) + (int64_t)c * Q * c_pitch,
+                                   (int64_t)(min(Q, p.seqlen - c * Q) - 1) * c_pitch + N * 2);
 #pragma unroll
         for (int k = 0; k < CI; ++k) {
             const int ins = wave * CI + k;
             const int t = ins * (64 / PRC) + lane / PRC;                // token within the chunk
             const int q = (lane % PRC) ^ (t & (PRC - 1));
-            load_to_lds(rsC, cld + ins * 1024, t * (int)c_pitch + q * 16, c * Q * (int)c_pitch);
+            load_to_lds(rsC, cld + ins * 1024, t * (int)c_pitch + q * 16, 0);
         }
     }
     request_head(0);
@@ -454,8 +459,8 @@ __global__ void __launch_bounds__(256, 1) scan_states_heads_kernel(const ScanPar
                 slo[ks][e] = pack_bf16(v[2 * e] - f0, v[2 * e + 1] - f1);
             }
         }
-        const auto rsO = make_rsrc((char *)p.out + esz * (b * p.so_b + h * p.so_h + p0 + 16 * wave),
-                                   ((int64_t)(p.seqlen - 1) * o_pitch + 16) * esz);
+        const auto rsO = make_rsrc((char *)p.out + esz * (b * p.so_b + h * p.so_h + p0 + 16 * wave + (int64_t)c * Q * o_pitch),
+                                   ((int64_t)(min(Q, p.seqlen - c * Q) - 1) * o_pitch + 16) * esz);
         const float *dal = (const float *)(dld + (i & 1) * 1024);
 
         // Software pipeline over the 16-token blocks: the C operands of block mb + 1 are read before the MFMAs of
@@ -485,12 +490,12 @@ __global__ void __launch_bounds__(256, 1) scan_states_heads_kernel(const ScanPar
                 ah = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[ks]), cf[ks], ah, 0, 0, 0);
                 al = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[ks]), cf[ks], al, 0, 0, 0);
             }
-            if (mb > 0) store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (c * Q + 16 * (mb - 1)) * (int)o_pitch, vprev);
+            if (mb > 0) store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (16 * (mb - 1)) * (int)o_pitch, vprev);
             // acc[r] = y[token 16 mb + i16][row 4 kg + r]: through LDS to (token lane / 4, 16-byte piece lane % 4)
             *(f32x4 *)owr = (ah + al) * sc;
             vprev = *(const f32x4 *)ord;
         }
-        store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (c * Q + 16 * (MBT - 1)) * (int)o_pitch, vprev);
+        store_y<PLAIN>(rsO, p.dt_out, p.accumulate, voff, (16 * (MBT - 1)) * (int)o_pitch, vprev);
     }
 }
 
@@ -541,8 +546,8 @@ bool scan_states_mfma_supported(const ScanParams &p)
     if ((p.sst_b | p.sst_c | p.sst_h | p.sst_p) % (p.dt_states == DT_F32 ? 4 : 8) != 0) return false;
     const int per16 = p.dt_out == DT_F32 ? 4 : 8;
     if ((p.so_b | p.so_l | p.so_h) % per16 != 0) return false;
-    // byte offsets inside one descriptor are 32-bit
-    if ((int64_t)p.seqlen * p.sC_l * 2 >= 0x7fffffffLL || (int64_t)p.seqlen * p.so_l * 4 >= 0x7fffffffLL) return false;
+    // byte offsets inside one descriptor are 32-bit; the descriptors of C and y cover one chunk
+    if ((int64_t)p.Q * p.sC_l * 2 >= 0x7fffffffLL || (int64_t)p.Q * p.so_l * (p.dt_out == DT_F32 ? 4 : 2) >= 0x7fffffffLL) return false;
     if ((int64_t)p.headdim * p.sst_p * 4 >= 0x7fffffffLL) return false;
     return (int64_t)p.batch * p.C * p.nheads * (p.headdim / 32) < 0x7fffffffLL;
 }

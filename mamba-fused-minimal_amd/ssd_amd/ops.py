@@ -36,7 +36,11 @@ def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
     return B, x, dt, dA_cumsum, seq_idx
 
 
-def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True, _clamp=True):
+def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
+    return _chunk_state_impl(B, x, dt, dA_cumsum, seq_idx, states, states_in_fp32, True)
+
+
+def _chunk_state_impl(B, x, dt, dA_cumsum, seq_idx, states, states_in_fp32, _clamp):
     # _clamp=False evaluates the decay as the reference's fused kernels do (no min(., 0), fused_globalbar.py:106)
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape

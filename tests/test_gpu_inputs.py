@@ -72,7 +72,7 @@ def test_unclamped_decay_on_every_kernel_family(ops, oracle, family):
     for clamp in (True, False):
         old = ops.set_token_split(split)
         try:
-            st = ops._chunk_state_fwd(_dev(d["B"]), _dev(d["x"]), _dev(d["dt"]), _dev(d["dA_cumsum"]), _clamp=clamp)
+            st = ops.ops._chunk_state_impl(_dev(d["B"]), _dev(d["x"]), _dev(d["dt"]), _dev(d["dA_cumsum"]), None, None, True, clamp)
             torch.cuda.synchronize()
         finally:
             ops.set_token_split(old)

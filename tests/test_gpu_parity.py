@@ -493,6 +493,35 @@ def test_chunk_scan_states_cfg2_row(ops, oracle):
     assert err <= 1e-30
 
 
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_chunk_scan_states_long_grouped(ops, oracle, out_dtype):
+    # The long grouped configuration at full size: seqlen * row pitch of y is 4.3 GB in fp32, past what one 32-bit
+    # buffer descriptor reaches, so C and y are addressed chunk by chunk.  The states come from the fused call; two
+    # heads of different groups are compared with the oracle, and the call must have run on the matrix-core kernels
+    # (the element-per-thread fallback would take seconds).
+    d = oracle.make_inputs(4)
+    dA = d["dA_cumsum"]
+    xd, Bd, dtd, dAd, Cd = map(_dev, (d["x"], d["B"], d["dt"], dA, d["C"]))
+    prev, _ = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, torch.float32)
+    del xd, Bd, dtd
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    y = ops._chunk_scan_states_fwd(Cd, prev, dAd, out_dtype=out_dtype)       # warm-up
+    ev[0].record()
+    y = ops._chunk_scan_states_fwd(Cd, prev, dAd, out_dtype=out_dtype)
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = ev[0].elapsed_time(ev[1])
+    print(f"[scan_states.cfg4.{out_dtype}] {ms * 1e3:.0f} us", flush=True)
+    assert ms < 20.0, "the matrix-core kernels take a few milliseconds at this size"
+    ratio = d["x"].shape[2] // d["B"].shape[2]
+    lowp = out_dtype != torch.float32
+    for h in (5, 127):
+        g = h // ratio
+        want = oracle.chunk_scan_states_ref(d["C"][:, :, g:g + 1], prev[:, :, h:h + 1].cpu(), dA[:, h:h + 1])
+        _check(f"scan_states.cfg4.h{h}", y[:, :, h:h + 1], want, *((1e-2, 1e-2) if lowp else (RTOL, ATOL)))
+
+
 # ------------------------------------------------------------------ the path inside a whole SSD forward
 @pytest.mark.parametrize("kw", [dict(), dict(nseq=4, L=900, init=True)], ids=["plain", "varlen-ragged-init"])
 def test_whole_ssd_forward_with_library_kernels(ops, oracle, kw):
