@@ -163,6 +163,26 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
 int ssd_fused_workspace_status(const void *workspace, void *stream);
 
 /*
+ * ssd_fused_chunk_state_passing_fwd_ws without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory or have it allocated on their
+ * behalf: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The ticket counters and
+ * flags live in a fixed 1 MiB array inside the library's own code object (one copy per GPU, held until the process
+ * ends); the call clears what it uses with a small fill launch and runs the chain kernel, whatever the problem size
+ * (the kernel choice of the other entry points is not made here: SSD_ERR_SHAPE for arguments that kernel does not
+ * cover -- it needs bf16 x / B, fp32 out / initial / final states, dstate 64 or 128, chunk 128 or 256 --,
+ * SSD_ERR_SCRATCH when batch * nheads * (headdim / 32) * nchunks + 64 flags do not fit the array, i.e. above 262 080
+ * (state tile, chunk) pairs).  Every call on a GPU shares that GPU's array: two calls whose kernels may overlap
+ * (different streams, different host threads) race on it and must be serialised by the caller.
+ * ssd_fused_static_status is ssd_fused_workspace_status for that array.
+ */
+int ssd_fused_chunk_state_passing_fwd_static(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                             const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                             const ssd_tensor *initial_states, const ssd_tensor *out,
+                                             const ssd_tensor *final_states, const ssd_dims *dims, int clamp,
+                                             void *stream);
+int ssd_fused_static_status(void *stream);
+
+/*
  * Which kernel family the three calls above would pick for these arguments: 1 = bf16 MFMA path,
  * 0 = generic FMA path (other element types or shapes the MFMA tiling does not cover), negative = rejected.
  * Pure host logic; launches nothing.

@@ -170,6 +170,34 @@ int run(const Params &p, bool fused, void *stream)
     return (int)e;
 }
 
+// Scratch for ssd_fused_chunk_state_passing_fwd_static: ticket counters, error word and flags of the chain kernel in
+// device memory that belongs to the library's code object -- every GPU the library runs on holds its own copy, at its
+// own address, until the process ends.  The name is a host-side handle, not a device address: the address is asked
+// for once per device (scratch_pointer) and only that pointer is handed to kernels.
+constexpr int kStaticScratchInts = 1 << 18;     // 1 MiB: header + one flag per (state tile, chunk)
+static __device__ __align__(256) int g_static_scratch[kStaticScratchInts];
+
+std::atomic<int *> g_scratch_ptr[64];
+
+// device address of g_static_scratch on the current device (nullptr + error code on failure)
+hipError_t scratch_pointer(int **ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) {
+        int *cached = g_scratch_ptr[dev].load(std::memory_order_acquire);
+        if (cached) { *ptr = cached; return hipSuccess; }
+    }
+    void *sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess) return e;
+    if (!sym) return hipErrorInvalidSymbol;
+    if (dev >= 0 && dev < 64) g_scratch_ptr[dev].store((int *)sym, std::memory_order_release);
+    *ptr = (int *)sym;
+    return hipSuccess;
+}
+
 // Whether the ticket / flag-chain kernel is the better fused kernel for a problem it covers: it keeps every compute
 // unit busy whatever the number of state tiles, at the price of reading each passed state back once.
 bool chain_preferred(const Params &p)
@@ -278,6 +306,36 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
     }
     if (kernel != SSD_KERNEL_AUTO) return SSD_ERR_SCRATCH;     // forced, but no workspace or not a shape it covers
     return run(p, true, stream);
+}
+
+int ssd_fused_chunk_state_passing_fwd_static(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                             const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                             const ssd_tensor *initial_states, const ssd_tensor *out,
+                                             const ssd_tensor *final_states, const ssd_dims *dims, int clamp,
+                                             void *stream)
+{
+    Params p;
+    int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, nullptr, out, final_states, dims, clamp);
+    if (rc) return rc;
+    if (!ssd::chain_supported(p)) return SSD_ERR_SHAPE;        // only the kernel that needs scratch is offered here
+    if (ssd_fused_workspace_bytes(dims) > sizeof(int) * (uint64_t)kStaticScratchInts) return SSD_ERR_SCRATCH;
+    rc = check_device();
+    if (rc) return rc;
+    int *scratch = nullptr;
+    const hipError_t e = scratch_pointer(&scratch);
+    if (e != hipSuccess) return (int)e;
+    p.ws = scratch;
+    return (int)ssd::launch_chain(p, compute_units(), 0, (hipStream_t)stream);
+}
+
+int ssd_fused_static_status(void *stream)
+{
+    int rc = check_device();
+    if (rc) return rc;
+    int *scratch = nullptr;
+    const hipError_t e = scratch_pointer(&scratch);
+    if (e != hipSuccess) return (int)e;
+    return ssd_fused_workspace_status(scratch, stream);
 }
 
 int ssd_fused_workspace_status(const void *workspace, void *stream)

@@ -14,7 +14,8 @@ _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
            "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes",
-           "ssd_fused_workspace_status", "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
+           "ssd_fused_workspace_status", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
+           "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
 class SsdTensor(ctypes.Structure):
@@ -64,6 +65,10 @@ def load():
     lib.ssd_fused_workspace_bytes.argtypes = [D]
     lib.ssd_fused_workspace_status.restype = ctypes.c_int
     lib.ssd_fused_workspace_status.argtypes = [vp, vp]
+    lib.ssd_fused_chunk_state_passing_fwd_static.restype = ctypes.c_int
+    lib.ssd_fused_chunk_state_passing_fwd_static.argtypes = [T, T, T, T, T, T, T, T, D, ctypes.c_int, vp]
+    lib.ssd_fused_static_status.restype = ctypes.c_int
+    lib.ssd_fused_static_status.argtypes = [vp]
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.restype = ctypes.c_int
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.argtypes = [T] * 11 + [D, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, vp]
     lib.ssd_query_path.restype = ctypes.c_int

@@ -157,6 +157,44 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     return out, final_states
 
 
+def _fused_chunk_state_state_passing_fwd_static(B, x, dt, dA_cumsum, out, final_states, initial_states=None, seq_idx=None,
+                                                _clamp=True):
+    """The fused call on the entry point that allocates nothing (ssd_fused_chunk_state_passing_fwd_static): the
+    caller brings ``out`` (b,C,H,P,N) fp32 and ``final_states`` (b,H,P,N) fp32, the tickets and flags live in a
+    fixed array inside the library, and this wrapper creates no tensor either (inputs must already have the types
+    and unit inner strides the kernel takes).  No counterpart in the reference.  Calls that may overlap on one GPU
+    race on that array."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size) and dA_cumsum.shape == dt.shape
+    assert out.shape == (batch, nchunks, nheads, headdim, dstate) and final_states.shape == (batch, nheads, headdim, dstate)
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen) and seq_idx.dtype == torch.int32
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+    _lib.require_device(x, "_fused_chunk_state_state_passing_fwd_static")
+    lib = _lib.load()
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    with torch.cuda.device(x.device):
+        rc = lib.ssd_fused_chunk_state_passing_fwd_static(
+            _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),
+            _lib.tensor_arg(seq_idx), _lib.tensor_arg(initial_states), _lib.tensor_arg(out),
+            _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, _stream(x))
+    _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_static")
+    return out, final_states
+
+
+def _fused_static_status(device=None):
+    """Waits for the current stream and returns 0, or -7 if a flag wait of the last
+    ssd_fused_chunk_state_passing_fwd_static launch on this device ran out."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    with torch.cuda.device(device):
+        return int(_lib.load().ssd_fused_static_status(ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)))
+
+
 def _fused_workspace_status(workspace):
     """Waits for the current stream and returns 0, or -7 if a flag wait of the last fused launch that used
     ``workspace`` ran out (ssd_fused_workspace_status)."""

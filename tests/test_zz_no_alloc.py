@@ -1,0 +1,75 @@
+"""GPU test of the entry point that allocates nothing (ssd_fused_chunk_state_passing_fwd_static), through the C ABI:
+its outputs against those of ssd_fused_chunk_state_passing_fwd_ws on the same inputs -- the same kernel with a
+caller-provided workspace --, on two calls in a row, the second with a smaller input, and against the CPU oracle
+(rtol 2e-3 / atol 1e-3).  Collected last: the scratch array is shared by every call of the process."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(t):
+    return None if t is None else t.cuda()
+
+
+def _pair(ops, oracle, kw, name):
+    d = oracle.make_inputs(2, **kw)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    init, seq = _dev(d["initial_states"]), _dev(d["seq_idx"])
+    b, L, H, P = d["x"].shape
+    N, C = d["B"].shape[-1], d["dt"].shape[2]
+    print(f"[{name}] x{tuple(d['x'].shape)} chunks={C} init={init is not None} seq={seq is not None}", flush=True)
+    # outputs poisoned: every element must be written by the call
+    out = torch.full((b, C, H, P, N), float("nan"), device="cuda")
+    fin = torch.full((b, H, P, N), float("nan"), device="cuda")
+    ops._fused_chunk_state_state_passing_fwd_static(*args, out, fin, initial_states=init, seq_idx=seq)
+    assert ops._fused_static_status() == 0
+    want_out, want_fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=init, seq_idx=seq,
+                                                                  _kernel=1)
+    torch.cuda.synchronize()
+    # the same kernel on the same inputs: the same bits
+    assert torch.equal(out, want_out), f"{name}: out differs, max {float((out - want_out).abs().max()):.3e}"
+    assert torch.equal(fin, want_fin), f"{name}: final_states differ"
+    ref_out, ref_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"],
+                                        seq_idx=d["seq_idx"])
+    for got, want in ((out, ref_out), (fin, ref_fin)):
+        err = (got.cpu() - want).abs()
+        assert int((err > 1e-3 + 2e-3 * want.abs()).sum()) == 0, f"{name}: max abs err {float(err.max()):.3e}"
+
+
+def test_static_scratch_entry_point_two_calls(oracle):
+    import ssd_amd
+    from ssd_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    _pair(ssd_amd, oracle, dict(b=2, L=8192, H=16), "static.first")                  # 32 chunks, initial states
+    _pair(ssd_amd, oracle, dict(b=1, L=2000, H=8, nseq=3), "static.second.smaller")  # fewer, ragged, packed sequences
+
+
+def test_static_scratch_rejects_what_does_not_fit():
+    from ssd_amd import _lib
+    lib = _lib.load()
+    # 262 144 ints: the header (64) plus one flag per (state tile, chunk).  b=8 L=131072 H=128 would need 1 M of them.
+    # The call is rejected before anything is launched, so the tensors only need plausible descriptions.
+    b, L, H, P, N, G, Q, C = 8, 131072, 128, 64, 128, 8, 256, 512
+    dims = _lib.dims_arg(b, L, H, P, N, G, Q, C)
+    assert lib.ssd_fused_workspace_bytes(dims) > 4 * (1 << 18)
+    anchor = torch.zeros(64, device="cuda")
+
+    def described(dtype, shape):
+        t = _lib.SsdTensor()
+        t.data = anchor.data_ptr()
+        t.dtype = dtype
+        stride = 1
+        for i in reversed(range(len(shape))):
+            t.stride[i] = stride
+            stride *= shape[i]
+        return t
+
+    none = _lib.tensor_arg(None)
+    rc = lib.ssd_fused_chunk_state_passing_fwd_static(
+        described(_lib.SSD_BF16, (b, L, H, P)), described(_lib.SSD_BF16, (b, L, G, N)), described(_lib.SSD_F32, (b, H, C, Q)),
+        described(_lib.SSD_F32, (b, H, C, Q)), none, none, described(_lib.SSD_F32, (b, C, H, P, N)),
+        described(_lib.SSD_F32, (b, H, P, N)), dims, 1, None)
+    assert rc == _lib.SSD_ERR_SCRATCH, rc
+    assert "workspace" in lib.ssd_status_string(rc).decode()
