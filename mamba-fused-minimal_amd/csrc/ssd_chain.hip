@@ -117,6 +117,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     struct Item {
         int valid, c, r, b, h, tile, p0;           // r: position of the chunk in its work item
         __amdgpu_buffer_rsrc_t rsx, rsB;
+        const char *xb, *Bb;                       // chunk 0 of the tile's x rows and of its group's B rows
         const float *dtp, *dap;
         const int32_t *sqb;
     };
@@ -137,10 +138,10 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         I.h = r1 - I.b * p.nheads;
         const int g = I.h / (p.nheads / p.ngroups);
         // descriptor of the chunk: base = its first token, extent = the tokens that exist
-        const char *xb = (const char *)p.x + 2 * (I.b * p.sx_b + I.h * p.sx_h) + (int64_t)I.c * Q * xrb;
-        const char *Bb = (const char *)p.B + 2 * (I.b * p.sB_b + g * p.sB_g) + (int64_t)I.c * Q * Brb;
-        I.rsx = make_rsrc(xb, I.valid ? (int64_t)(L - I.c * Q) * xrb : 0);
-        I.rsB = make_rsrc(Bb, I.valid ? (int64_t)(L - I.c * Q) * Brb : 0);
+        I.xb = (const char *)p.x + 2 * (I.b * p.sx_b + I.h * p.sx_h);
+        I.Bb = (const char *)p.B + 2 * (I.b * p.sB_b + g * p.sB_g);
+        I.rsx = make_rsrc(I.xb + (int64_t)I.c * Q * xrb, I.valid ? (int64_t)(L - I.c * Q) * xrb : 0);
+        I.rsB = make_rsrc(I.Bb + (int64_t)I.c * Q * Brb, I.valid ? (int64_t)(L - I.c * Q) * Brb : 0);
         I.dtp = p.dt + I.b * p.sdt_b + I.h * p.sdt_h + (int64_t)I.c * p.sdt_c;
         I.dap = p.dacs + I.b * p.sda_b + I.h * p.sda_h + (int64_t)I.c * p.sda_c;
         I.sqb = HAS_SEQ ? p.seq + I.b * p.ssq_b : nullptr;
@@ -153,11 +154,8 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             (void)t_cur;
             J.c = I.c + 1;
             J.r = I.r + 1;
-            const int g = I.h / (p.nheads / p.ngroups);
-            const char *xb = (const char *)p.x + 2 * (I.b * p.sx_b + I.h * p.sx_h) + (int64_t)J.c * Q * xrb;
-            const char *Bb = (const char *)p.B + 2 * (I.b * p.sB_b + g * p.sB_g) + (int64_t)J.c * Q * Brb;
-            J.rsx = make_rsrc(xb, (int64_t)(L - J.c * Q) * xrb);
-            J.rsB = make_rsrc(Bb, (int64_t)(L - J.c * Q) * Brb);
+            J.rsx = make_rsrc(I.xb + (int64_t)J.c * Q * xrb, (int64_t)(L - J.c * Q) * xrb);
+            J.rsB = make_rsrc(I.Bb + (int64_t)J.c * Q * Brb, (int64_t)(L - J.c * Q) * Brb);
             J.dtp = I.dtp + p.sdt_c;
             J.dap = I.dap + p.sda_c;
             return J;
@@ -442,8 +440,8 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             raise_flag(flag + c0 + n);
         }
         // ... then the states inside the item, which nobody waits for.  (Spreading these stores over the steps of the
-        // next item was measured: 250 us instead of 215 at b=4 L=8192 H=80 -- memory operations complete in order, so
-        // every later wait for a load also waits for the stores issued before it, and a store is acknowledged late.)
+        // next item was measured: 250 us instead of 215 at b=4 L=8192 H=80; the non-temporal hint on these stores:
+        // 220 instead of 213.)
         static_for<R>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             if (j < n - 1) store_chunk(j, held[j], 0);
@@ -560,9 +558,13 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l1, acc[it][1], 0, 0, 0);
-            // next step's x operands, one or two eighths per iteration
+            // next step's x operands, spread over the iterations after the first (their LDS reads, issued at the top
+            // of the step, get the first iteration to arrive)
+            {
+                constexpr int e0 = it == 0 ? 0 : (it - 1) * 8 / (NT - 1), e1 = it == 0 ? 0 : it * 8 / (NT - 1);
 #pragma unroll
-            for (int e = it * 8 / NT; e < (it + 1) * 8 / NT; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
+                for (int e = e0; e < e1; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
+            }
             if (it == 0) { load_x(rsx, xp0, s3, 0); load_x(rsx, xp0, s3, 1); }
             if (it >= NT - kAhead && it < NT - kAhead + NTW) load_B(rsB, s3, wave * NTW + (it - (NT - kAhead)));
             if (s == 1 && it == NT - 1 && nxt.valid) mnext = load_meta(nxt);
