@@ -13,6 +13,13 @@
  * dA_cumsum[..., -1]) are passed without copies.  The innermost stride of x, B, states, out,
  * initial_states and final_states must be 1.
  *
+ * Threads: an entry point may be called from any host thread; a call holds no state of its own beyond its
+ * arguments.  What the library keeps per process is atomic: a cache of device properties, a per-device record of
+ * which kernels have been given their LDS size, and the three ssd_set_* hooks below, which are process-wide test and
+ * tuning knobs (a value set in one thread changes the kernel choice of later calls in every thread, never their
+ * results beyond rounding).  Calls that overlap in time must not share a workspace (ssd_fused_opts) or the static
+ * scratch (ssd_fused_chunk_state_passing_fwd_static).
+ *
  * Replaces, in the reference repository (RishiAstra/mamba-fused-minimal):
  *   ssd_chunk_state_fwd                -> kernels/ssd_chunk_state.py:202-232 (_chunk_state_fwd) and the
  *                                         Triton kernel it launches, kernels/ssd_chunk_state.py:97-173

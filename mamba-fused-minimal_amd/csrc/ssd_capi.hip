@@ -138,10 +138,13 @@ Params with_states_in_out(const Params &p)
     return q;
 }
 
-int run(const Params &p, bool fused, void *stream)
+int run(const Params &p_in, bool fused, void *stream)
 {
     int rc = check_device();
     if (rc) return rc;
+    Params p = p_in;
+    p.n_cu = compute_units();
+    const int64_t n_cu = p.n_cu > 0 ? p.n_cu : 256;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
     // Fused launch: with at least two state tiles per compute unit the four-tiles-per-workgroup kernel wins (B is
@@ -149,21 +152,21 @@ int run(const Params &p, bool fused, void *stream)
     // kernel, which puts four waves on every tile, has the shorter chunk.
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
     const int g_forced_split = ::g_forced_split.load(std::memory_order_relaxed);      // one value for the whole choice
-    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 512)) && ssd::quad_supported(p))
+    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 2 * n_cu)) && ssd::quad_supported(p))
         e = ssd::launch_quad(p, s);
-    else if (fused && !p.states && g_forced_split == 0 && tiles < 512 && (int64_t)tiles * p.C >= 8192 &&
+    else if (fused && !p.states && g_forced_split == 0 && tiles < 2 * n_cu && (int64_t)tiles * p.C >= 32 * n_cu &&
              p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p))) {
         // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
         // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
         // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
         e = launch_pair(with_states_in_out(p), s);
-    } else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8192)) &&
+    } else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 32 * n_cu)) &&
                pair_supported(p)) {
         // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
         // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
         // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
         e = launch_pair(p, s);
-    } else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 2048)) &&
+    } else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8 * n_cu)) &&
              ssd::quad_chunk_state_supported(p))
         e = ssd::launch_quad_chunk_state(p, s);
     else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);

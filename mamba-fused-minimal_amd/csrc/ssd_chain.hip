@@ -76,6 +76,10 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     constexpr int Q = 32 * SPC;
     constexpr int kRing = ring_of<SPC>(), kDist = kRing - 1;
     static_assert(kDist < SPC, "the requests of a step reach into the next chunk at most");
+    // the step loop's vector-memory queue, replayed at compile time (ssd_tile.h): 2 x requests and NT / 4 B requests
+    // per step, no stores inside the loop
+    constexpr schedule::Loop kLoop{2, NT / 4, 0, SPC, kDist, kRing};
+    static_assert(schedule::slots_ok(kLoop), "ring slots are reused too early");
     constexpr int TPL = Q / 64;         // tokens per lane when an item's weights are computed (2 or 4)
     constexpr int NTW = NT / 4;         // B tile blocks (32 tokens x 16 columns, 1 KB) a wave fetches per step
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -488,6 +492,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     u32x2 blo[4], bhi[4];
     {
         // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
+        static_assert(schedule::wait_prologue(kLoop) == (kDist - 1) * (2 + NTW), "prologue wait");
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 1) * (2 + NTW)));
         __builtin_amdgcn_s_barrier();   // ... and every other wave's blocks of step 0
         asm volatile("" ::: "memory");
@@ -517,6 +522,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         constexpr int s = decltype(sc)::value;
         // x rows of step + 1 (this wave's own, requested two steps ago): behind them came the B requests of that
         // step and all requests of the steps s + 2 - kDist .. s - 1
+        static_assert(schedule::wait_x(kLoop, s) == NTW + (kDist - 2) * (2 + NTW), "wait for the x rows of step + 1");
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(NTW + (kDist - 2) * (2 + NTW)));
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
@@ -545,6 +551,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 // ago) have landed once only the requests of step - 1 and the x requests of this step are
                 // outstanding; the barrier publishes every wave's blocks.  It also tells that all waves are through
                 // with the tile of step - 1, whose ring slot the B requests below overwrite.
+                static_assert(schedule::wait_b(kLoop, s) == (kDist - 2) * (2 + NTW) + 2, "wait for the B blocks of step + 1");
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 2) * (2 + NTW) + 2));
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");

@@ -623,7 +623,7 @@ hipError_t launch_mfma(const Params &p_in, bool fused, hipStream_t s)
     // unfused launch, whose (batch, chunk, head, slice) items are plentiful.  The fused launch walks the chunks of
     // a tile serially with the running state in registers; there four waves win (2-wave workgroups spill and a
     // tile's chunk takes twice as long), 285 vs 361 us at b=4 L=8192 H=80.
-    int wv = (!fused && p.n_items > 512) ? 2 : 4;
+    int wv = (!fused && p.n_items > 2 * (p.n_cu > 0 ? p.n_cu : 256)) ? 2 : 4;     // more than two tiles per compute unit
     const int forced = g_force_split.load(std::memory_order_relaxed);
     if (forced == 2 || forced == 4) wv = forced;
     const int nb = p.dstate / 16, q128 = p.Q / 128;     // chunk 128 or 256

@@ -38,6 +38,7 @@ struct Params {
     int *ws;              // ticket counter, error word and flags of the ticket / flag-chain kernel
     int spin_limit;       // polls after which a wave of that kernel stops waiting for a flag
     int n_xcd;            // XCDs (L2 caches) the units of that kernel are dealt to
+    int n_cu;             // compute units of the device (0: not known, the launchers then assume 256 in 8 XCDs)
 };
 
 // State passing on a flattened state axis.

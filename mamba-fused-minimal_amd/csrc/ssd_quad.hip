@@ -25,6 +25,7 @@
 // One s_barrier per step orders the shared ring: a wave passes it after its own part of the step's B tile has
 // landed and after it has finished reading the previous step's tile.
 #include "ssd_params.h"
+#include "ssd_tile.h"      // schedule:: the compile-time model of the step loop's memory queue
 
 #include <utility>
 
@@ -118,11 +119,11 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     char *stage = lds + kRing * NT * 1024 + 4 * wave_lds<NT, SPC>() + wave * kStage;
 
     // Work item -> (batch, head, row slice); the four items of a workgroup share batch and group (checked on the
-    // host).  Consecutive workgroups sit on the same XCD (workgroups are dealt round-robin over the 8 XCDs), so a
-    // batch's B is fetched from HBM by one or two L2 slices only.
+    // host).  Consecutive workgroups sit on the same XCD (workgroups are dealt round-robin over the p.n_xcd XCDs), so
+    // a batch's B is fetched from HBM by one or two L2 slices only.
     const int n_wg = p.n_items >> 2, n_seg = CO ? p.n_seg : 1;
-    const int per_xcd = (n_wg * n_seg + 7) >> 3;                         // workgroups per XCD
-    const int vwg = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    const int per_xcd = (n_wg * n_seg + p.n_xcd - 1) / p.n_xcd;          // workgroups per XCD
+    const int vwg = (int)(blockIdx.x % p.n_xcd) * per_xcd + (int)(blockIdx.x / p.n_xcd);
     if (vwg >= n_wg * n_seg) return;                                     // whole workgroup: no barrier is skipped
     int wg = vwg, c0 = 0, c1 = p.C;
     if (CO) {
@@ -414,6 +415,11 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     // vector-memory operations of one store_state, at least (a 16-bit `out` takes NT stores, a 32-bit one 2 NT; the
     // waits below may count fewer operations than were issued, never more)
     constexpr int kStores = F32IO ? 2 * NT : NT;
+    // the loop's vector-memory queue, replayed at compile time: 2 x requests and NT / 4 B requests per step, the state
+    // stores at the first step of every chunk
+    constexpr tile::schedule::Loop kLoop{2, NT / 4, kStores, SPC, kDist, kRing};
+    static_assert(tile::schedule::slots_ok(kLoop), "ring slots are reused too early");
+    static_assert(tile::schedule::wait_prologue(kLoop) == (kDist - 1) * (2 + NTW), "prologue wait");
     u32x2 blo[4], bhi[4];
     {
         // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
@@ -444,6 +450,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         // x rows of step + 1 (this wave's own, requested two steps ago): behind them came the B requests of that
         // step and all requests of the steps s + 2 - kDist .. s - 1 (with the state stores, if step 0 is among them)
         constexpr bool st_top = s >= 1 && s <= kDist - 2;         // step 0 among them
+        static_assert(tile::schedule::wait_x(kLoop, s) == NTW + (kDist - 2) * (2 + NTW) + (st_top ? kStores : 0),
+                      "wait for the x rows of step + 1");
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(NTW + (kDist - 2) * (2 + NTW) + (st_top ? kStores : 0)));
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
@@ -497,6 +505,8 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
                 // also tells that all waves are through with the tile of step - 1, whose ring slot the B requests
                 // below overwrite.
                 constexpr bool st_mid = s < kDist - 1;       // step 0 among the steps s + 2 - kDist .. s
+                static_assert(tile::schedule::wait_b(kLoop, s) == (kDist - 2) * (2 + NTW) + 2 + (st_mid ? kStores : 0),
+                              "wait for the B blocks of step + 1");
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 2) * (2 + NTW) + 2 + (st_mid ? kStores : 0)));
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
@@ -610,7 +620,7 @@ static hipError_t launch_quad_k(const Params &p, dim3 grid, hipStream_t s)
 template <int NT, int SPC, bool CO>
 static hipError_t launch_quad_t(const Params &p, hipStream_t s)
 {
-    dim3 grid((((p.n_items >> 2) * (CO ? p.n_seg : 1) + 7) / 8) * 8);
+    dim3 grid((((p.n_items >> 2) * (CO ? p.n_seg : 1) + p.n_xcd - 1) / p.n_xcd) * p.n_xcd);
     const bool f32io = CO ? p.dt_states == DT_F32 : p.dt_out == DT_F32 && (!p.init || p.dt_init == DT_F32);
     if (p.seq) return f32io ? launch_quad_k<NT, SPC, true, true, CO>(p, grid, s) : launch_quad_k<NT, SPC, true, false, CO>(p, grid, s);
     return f32io ? launch_quad_k<NT, SPC, false, true, CO>(p, grid, s) : launch_quad_k<NT, SPC, false, false, CO>(p, grid, s);
@@ -631,6 +641,8 @@ hipError_t launch_quad(const Params &p_in, hipStream_t s)
     Params p = p_in;
     p.n_items = p.batch * p.nheads * (p.headdim / 32);
     if (p.n_items <= 0) return hipSuccess;
+    if (p.n_cu <= 0) p.n_cu = 256;
+    p.n_xcd = p.n_cu >= 32 ? p.n_cu / 32 : 1;       // an XCD is 32 compute units on this part
     return launch_quad_c<false>(p, s);
 }
 
@@ -643,6 +655,8 @@ hipError_t launch_quad_chunk_state(const Params &p_in, hipStream_t s)
     Params p = p_in;
     p.n_items = p.batch * p.nheads * (p.headdim / 32);
     if (p.n_items <= 0 || p.C <= 0) return hipSuccess;
+    if (p.n_cu <= 0) p.n_cu = 256;
+    p.n_xcd = p.n_cu >= 32 ? p.n_cu / 32 : 1;
     // Chunks per workgroup.  Measured times follow  (workgroups per compute unit, rounded up) x (chunks per
     // workgroup + 0.4): a workgroup's first requests have nothing to hide behind, which costs about 0.4 of a chunk,
     // and the compute unit with the most workgroups finishes last (b=4 L=8192 H=80: 190 / 162 / 160 / 177 / 219 us
@@ -652,7 +666,7 @@ hipError_t launch_quad_chunk_state(const Params &p_in, hipStream_t s)
         double best = 0;
         for (int k = 1; k <= p.C; ++k) {
             const int nseg = (p.C + k - 1) / k;
-            const int per_cu = ((p.n_items >> 2) * nseg + 255) / 256;
+            const int per_cu = ((p.n_items >> 2) * nseg + p.n_cu - 1) / p.n_cu;
             const double t = per_cu * (k + 0.4);
             if (cps <= 0 || t < best) { best = t; cps = k; }
         }

@@ -50,6 +50,71 @@ __device__ __forceinline__ void store4_f32(__amdgpu_buffer_rsrc_t rs, int voff, 
     asm volatile("s_nop 3" ::"v"(q) : "memory");
 }
 
+
+// Compile-time model of the vector-memory queue of the step loops that stream x and B through LDS rings
+// (ssd_quad.hip, ssd_chain.hip).  Per 32-token step t these kernels issue, in this program order,
+//     [st state stores]     top of the step, only where t is the first step of a chunk and the kernel stores there
+//     xr requests           the x rows of step t + dist                     (MFMA iteration 0)
+//     -- wait W2, s_barrier --                                              (MFMA iteration NT - kAhead)
+//     bw requests           this wave's B blocks of step t + dist
+// after a prologue that issues (xr, bw) for the steps 0 .. dist - 1, and they wait
+//     W0, end of the prologue:   this wave's B blocks of step 0 have landed
+//     W1, top of step t (before its stores):   the x rows of step t + 1 have landed
+//     W2, iteration NT - kAhead of step t:     this wave's B blocks of step t + 1 have landed.
+// Memory operations complete in the order they were issued, so "X has landed" is "at most n operations are
+// outstanding" with n = the number issued after X.  replay() walks the program order and counts that number for every
+// wait; the kernels static_assert their s_waitcnt immediates against it (operations the model leaves out -- decay
+// inputs, tickets, a chain step -- are issued after X or complete before it, and only make a wait longer).
+namespace schedule {
+
+struct Loop { int xr, bw, st, spc, dist, ring; };    // st: stores at a chunk's first step (0 = none)
+constexpr int kSteps = 48;                           // steps replayed: several chunks past the prologue
+struct Waits { int w0; int w1[kSteps]; int w2[kSteps]; };
+
+constexpr Waits replay(Loop k)
+{
+    Waits r{};
+    int last_x[kSteps + 16] = {}, last_b[kSteps + 16] = {};
+    int n = 0;      // operations issued so far
+    for (int t = 0; t < k.dist; ++t) {
+        n += k.xr; last_x[t] = n - 1;
+        n += k.bw; last_b[t] = n - 1;
+    }
+    r.w0 = n - 1 - last_b[0];
+    for (int t = 0; t < kSteps; ++t) {
+        r.w1[t] = n - 1 - last_x[t + 1];
+        if (k.st > 0 && t % k.spc == 0) n += k.st;
+        n += k.xr; last_x[t + k.dist] = n - 1;
+        r.w2[t] = n - 1 - last_b[t + 1];
+        n += k.bw; last_b[t + k.dist] = n - 1;
+    }
+    return r;
+}
+// the largest count that is safe for step s of every chunk (the fewest operations behind the one needed)
+constexpr int wait_x(Loop k, int s)
+{
+    const Waits r = replay(k);
+    int m = r.w1[s];
+    for (int t = s; t < kSteps; t += k.spc) m = r.w1[t] < m ? r.w1[t] : m;
+    return m;
+}
+constexpr int wait_b(Loop k, int s)
+{
+    const Waits r = replay(k);
+    int m = r.w2[s];
+    for (int t = s; t < kSteps; t += k.spc) m = r.w2[t] < m ? r.w2[t] : m;
+    return m;
+}
+constexpr int wait_prologue(Loop k) { return replay(k).w0; }
+// Ring slots.  The request for step t + dist, issued in step t, overwrites the slot of step t + dist - ring.  x: a
+// wave reads the rows of step u at the top of step u - 1, so u = t + dist - ring must satisfy u - 1 < t.  B: every
+// wave has consumed the tile of step u by the end of step u, and the requests of step t follow that step's barrier,
+// so u < t.  Both hold with a ring one longer than the distance; requests must not reach past the next chunk, and
+// the slot of a step must not depend on the chunk.
+constexpr bool slots_ok(Loop k) { return k.ring == k.dist + 1 && k.dist < k.spc && k.spc % k.ring == 0 && k.spc <= kSteps / 3; }
+
+}  // namespace schedule
+
 // bf16 hi / lo halves of the scaled x operand of one 32-token step: [row parity][token pair]
 struct Frag { uint32_t hi[2][4], lo[2][4]; };
 

@@ -83,6 +83,57 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_set_segment_chunks(-1) == -2 and lib.ssd_set_segment_chunks(3) == 0 and lib.ssd_set_segment_chunks(0) == 3
 
 
+def test_argument_validation_from_two_threads_with_different_hooks(lib):
+    # The three ssd_set_* hooks are process-wide atomics and everything else is per call: two host threads that keep
+    # setting different hook values while they call the argument-validation paths (which return before any device
+    # work) must see the same status codes as a single thread, workspace sizes that depend on the dims alone, and
+    # from every hook only values that one of the threads has stored (ctypes drops the GIL during the calls).
+    import threading
+    from ssd_amd import _lib
+    T = _lib.tensor_arg
+    x = torch.zeros(1, 256, 2, 64, dtype=torch.bfloat16)
+    B = torch.zeros(1, 256, 1, 128, dtype=torch.bfloat16)
+    dt = torch.zeros(1, 256, 2)
+    A = torch.zeros(2)
+    o = torch.zeros(1, 2, 1, 256)
+    good = _lib.dims_arg(1, 256, 2, 64, 128, 1, 256, 1)
+    bad = _lib.dims_arg(1, 256, 3, 64, 128, 2, 256, 1)
+    big = _lib.dims_arg(4, 8192, 80, 64, 128, 1, 256, 32)
+    want_ws = lib.ssd_fused_workspace_bytes(big)
+    assert want_ws == 4 * (64 + 4 * 80 * 2 * 32)
+    settings = {"a": (2, 3, 1), "b": (4, 5, 2)}
+    seen = {"split": {0, 2, 4}, "segment": {0, 3, 5}, "scan": {0, 1, 2}}
+    errors = []
+
+    def worker(name):
+        split, segment, scan = settings[name]
+        try:
+            for _ in range(300):
+                for hook, value, key in ((lib.ssd_set_token_split, split, "split"),
+                                         (lib.ssd_set_segment_chunks, segment, "segment"),
+                                         (lib.ssd_set_scan_kernel, scan, "scan")):
+                    old = hook(value)
+                    assert old in seen[key], (key, old)
+                assert lib.ssd_query_path(T(x), T(B), good) == 1
+                assert lib.ssd_query_path(T(x), T(B), bad) == -2
+                assert lib.ssd_query_path(T(None), T(B), good) == -1
+                assert lib.ssd_chunk_cumsum_fwd(T(dt), T(A), T(None), T(o), T(o), 1, 256, 2, 0, 0, 0.0, 1.0, None) == -2
+                assert lib.ssd_fused_workspace_bytes(big) == want_ws
+                assert lib.ssd_fused_chunk_state_passing_fwd_ws(T(x), T(B), T(None), T(None), T(None), T(None), T(None),
+                                                                T(None), T(None), good, 1, None, None) == -1
+                assert lib.ssd_set_token_split(3) == -2
+        except BaseException as e:      # report in the main thread
+            errors.append((name, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(n,)) for n in settings]
+    try:
+        for t in threads: t.start()
+        for t in threads: t.join()
+    finally:
+        lib.ssd_set_token_split(0); lib.ssd_set_segment_chunks(0); lib.ssd_set_scan_kernel(0)
+    assert not errors, errors
+
+
 def test_signatures_match_reference_call_surface():
     import ssd_amd
     sig = lambda f: list(inspect.signature(f).parameters)
