@@ -369,6 +369,53 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             for (int k = 0; k < 2 * NT; ++k) store4_f32(rs, row * pitch + col, (k & 1) * pitch + 16 * (k >> 1), v[k], aux);
         };
 
+        // held[j] <- exp(dA_j) [same sequence] held[j - 1] + held[j] for the chunks jb < j < je
+        auto carry_on = [&](int jb, int je) {
+            static_for<R>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if (j > jb && j < je) {
+                    const float sc = scale[j];
+#pragma unroll
+                    for (int k = 0; k < 2 * NT; ++k) {
+                        const f32x4 pv = held[j > 0 ? j - 1 : 0][k];
+                        held[j][k] = (f32x4){__builtin_fmaf(pv.x, sc, held[j][k].x), __builtin_fmaf(pv.y, sc, held[j][k].y),
+                                             __builtin_fmaf(pv.z, sc, held[j][k].z), __builtin_fmaf(pv.w, sc, held[j][k].w)};
+                    }
+                }
+            });
+        };
+        // the state the next item waits for: stored, acknowledged (by the L2 both sides share, or by memory), flagged.
+        // (Letting the next chunk's first wait for its own x rows stand in for the wait here -- memory operations
+        // complete in order -- saves it but raises the flag later: no gain at b=4 L=8192 H=80, and slower where the
+        // chain sets the pace: 1.19 ms instead of 1.10 ms at L=131072 H=128.)
+        auto hand_on = [&]() {
+            static_for<R>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if (j == n - 1) store_chunk(j, held[j], kAux);
+            });
+            if (c0 + n < C) {
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                asm volatile("" ::: "memory");
+                raise_flag(flag + c0 + n);
+            }
+        };
+        // A sequence that starts at chunk jz > 0 of the item (decay zero) cuts the item in two: the states from jz on do
+        // not depend on the state entering the item, so they are finished and handed on before this wave waits for
+        // its own predecessor -- with packed sequences the chain then is as long as a sequence, not as the batch row.
+        int jz = 0;
+        if (HAS_SEQ) {
+            static_for<R>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if (j >= 1 && j < n && scale[j] == 0.f) jz = j;
+            });
+        }
+        const int head = jz > 0 ? jz : n;           // chunks [0, head) depend on the state entering the item
+        if (jz > 0) {
+            carry_on(jz, n);
+            hand_on();
+        }
+
         if (use_prev && c0 > 0) {
             // out[:, c0] of this tile is complete once its flag is up
             int polls = 0;
@@ -393,19 +440,12 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                                                          4 * ((k & 1) * pitch_prev + 16 * (k >> 1)), kAux));
             }
             if (use_prev) {
-                // the recurrence over the item's chunks, in place: held[j] becomes the state after chunk c0 + j
-                static_for<R>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    if (j < n) {
-                        const float sc = scale[j];
+                // the recurrence enters the item: held[0] becomes the state after chunk c0
+                const float sc = scale[0];
 #pragma unroll
-                        for (int k = 0; k < 2 * NT; ++k) {
-                            const f32x4 pv = j == 0 ? s[k] : held[j > 0 ? j - 1 : 0][k];
-                            held[j][k] = (f32x4){__builtin_fmaf(pv.x, sc, held[j][k].x), __builtin_fmaf(pv.y, sc, held[j][k].y),
-                                                 __builtin_fmaf(pv.z, sc, held[j][k].z), __builtin_fmaf(pv.w, sc, held[j][k].w)};
-                        }
-                    }
-                });
+                for (int k = 0; k < 2 * NT; ++k)
+                    held[0][k] = (f32x4){__builtin_fmaf(s[k].x, sc, held[0][k].x), __builtin_fmaf(s[k].y, sc, held[0][k].y),
+                                         __builtin_fmaf(s[k].z, sc, held[0][k].z), __builtin_fmaf(s[k].w, sc, held[0][k].w)};
             }
             if (c0 == 0) {
 #pragma unroll
@@ -413,39 +453,13 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                     store4_f32(make_rsrc(outb, slice_out * 4), row * (int)p.so_p + col, (k & 1) * (int)p.so_p + 16 * (k >> 1), s[k], 0);
             }
         }
-        if (!use_prev) {
-            // the item starts a sequence: its first state is its first chunk state
-            static_for<R>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                if (j >= 1 && j < n) {
-                    const float sc = scale[j];
-#pragma unroll
-                    for (int k = 0; k < 2 * NT; ++k) {
-                        const f32x4 pv = held[j > 0 ? j - 1 : 0][k];
-                        held[j][k] = (f32x4){__builtin_fmaf(pv.x, sc, held[j][k].x), __builtin_fmaf(pv.y, sc, held[j][k].y),
-                                             __builtin_fmaf(pv.z, sc, held[j][k].z), __builtin_fmaf(pv.w, sc, held[j][k].w)};
-                    }
-                }
-            });
-        }
-        // the state the next item waits for first ...
-        static_for<R>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            if (j == n - 1) store_chunk(j, held[j], kAux);
-        });
-        if (c0 + n < C) {
-            // ... its stores have been acknowledged (by the L2 both sides share, or by memory) before the flag is raised.
-            // (Letting the next chunk's first wait for its own x rows stand in for this one -- memory operations
-            // complete in order -- saves the wait but raises the flag later: no gain at b=4 L=8192 H=80, and slower
-            // where the chain sets the pace: 1.19 ms instead of 1.10 ms at L=131072 H=128.)
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            asm volatile("" ::: "memory");
-            raise_flag(flag + c0 + n);
-        }
-        // ... then the states inside the item, which nobody waits for.  (Spreading these stores over the steps of the
-        // next item was measured: 250 us instead of 215 at b=4 L=8192 H=80; the non-temporal hint on these stores:
-        // 220 instead of 213.)
+        // ... and runs through its chunks, in place: held[j] becomes the state after chunk c0 + j (an item that starts
+        // a sequence starts from its first chunk state)
+        carry_on(0, head);
+        if (jz == 0) hand_on();
+        // the states inside the item, which nobody waits for.  (Spreading these stores over the steps of the next item
+        // was measured: 250 us instead of 215 at b=4 L=8192 H=80; the non-temporal hint on these stores: 220
+        // instead of 213.)
         static_for<R>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             if (j < n - 1) store_chunk(j, held[j], 0);
@@ -453,10 +467,18 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     };
 
     // ---- tickets ---------------------------------------------------------------------------------------------
+    // Tickets are worked on in the order they are drawn only if every workgroup draws one per item: two tickets drawn
+    // together at the start would put the second a whole item later than its neighbours' first ones, and the items
+    // that depend on it (same unit, next chunks: a smaller ticket distance than there are workgroups when units are
+    // few) would all be waiting by then.  So a workgroup starts with one ticket; the second is drawn while the first
+    // chunk of the first item runs and the third while its second chunk runs (below), after that one per item.  Only
+    // a first item of a single chunk needs its successor from its first steps on and draws it here.
     if (threadIdx.x == 0) {
-        const int t = __hip_atomic_fetch_add(ws_ticket, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int t = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int c_first = (t < total ? t / n_units : 0) * R;
+        const bool single = !(R > 1 && c_first + 1 < C);
         tq[0] = t;
-        tq[1] = t + 1;
+        tq[1] = single ? __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -1;
     }
     // rows past the end of the sequence are not fetched and leave their LDS slots untouched; their weight is zero,
     // so the slots only have to hold finite numbers
@@ -469,6 +491,8 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     __builtin_amdgcn_s_barrier();
     // the tickets of the current and of the next item; the one after that is drawn while the current item runs
     int t_cur = __builtin_amdgcn_readfirstlane(tq[0]), t_nxt = __builtin_amdgcn_readfirstlane(tq[1]);
+    bool second_late = t_nxt < 0;                // the second ticket is still to be drawn (first item only)
+    if (second_late) t_nxt = total;              // no item; not looked at before the ticket is there
     Item cur = decode(t_cur, 0);
     Item nxt = successor(cur, t_cur, t_nxt);
     if (!cur.valid) return;                      // whole workgroup: no barrier is skipped
@@ -528,9 +552,11 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         uint32_t xr[8]; float wv[8];
         if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
         else read_operands(0, ws ^ 1, xr, wv);
-        if (s == 0 && cur.r == 0 && threadIdx.x == 0)
+        if (s == 0 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
             t_new = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (s == SPC - 2 && cur.r == 0 && threadIdx.x == 0) tq[2] = t_new;     // published by this step's barrier
+        // published by this step's barrier: the ticket after next, or (first item) the next one and then that
+        if (s == SPC - 2 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
+            tq[second_late && cur.r == 0 ? 1 : 2] = t_new;
         // requests of this step: x rows and this wave's B blocks of step + 3 (this item or the next)
         const auto rsB = s + kDist < SPC ? cur.rsB : nxt.rsB;
         const auto rsx = s + kDist < SPC ? cur.rsx : nxt.rsx;
@@ -594,11 +620,13 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         }
         park(cur, mcur);
         zero_acc();
+        if (second_late && cur.r == 0) t_nxt = __builtin_amdgcn_readfirstlane(tq[1]);     // drawn during this chunk
         if (!(cur.r + 1 < R && cur.c + 1 < C)) {
             // the item's last chunk: the chain step, then the tickets move up
             chain_step(cur);
             t_cur = t_nxt;
             t_nxt = __builtin_amdgcn_readfirstlane(tq[2]);
+            second_late = false;
         }
         mcur = mnext;
         cur = nxt;
