@@ -74,6 +74,21 @@ def test_chain_kernel_variants(ops, oracle, kw, kernel, r):
     _chain_case(ops, oracle, oracle.make_inputs(1, **base), kernel, r, f"chain.k{kernel}.r{r}")
 
 
+@pytest.mark.parametrize("r", [2, 4])
+@pytest.mark.parametrize("kernel", [LOCAL, GLOBAL], ids=["local", "global"])
+def test_chain_items_cut_by_sequence_starts(ops, oracle, kernel, r):
+    # Sequence starts placed at every position inside a work item: in chunk 1 (mid-chunk), in chunks 6 and 7 (two in one
+    # item, one of them on a chunk's first token), in chunk 11 (the item's last chunk) and none in the last item.  The
+    # states behind the last start of an item are handed on before the item has seen its predecessor's state.
+    d = oracle.make_inputs(1, b=2, L=4096, H=8, init=True)
+    starts = [256 + 100, 6 * 256, 7 * 256 + 255, 11 * 256 + 17]
+    ids = torch.zeros(4096, dtype=torch.int32)
+    for s0 in starts:
+        ids[s0:] += 1
+    d["seq_idx"] = ids.reshape(1, -1).expand(2, -1).contiguous()
+    _chain_case(ops, oracle, d, kernel, r, f"chain.cut.k{kernel}.r{r}")
+
+
 @pytest.mark.timeout(600)
 @pytest.mark.parametrize("cfg", [2, 3], ids=["cfg2", "cfg3"])
 def test_chain_kernel_at_benchmark_configs(ops, oracle, cfg):
