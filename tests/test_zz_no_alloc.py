@@ -73,3 +73,39 @@ def test_static_scratch_rejects_what_does_not_fit():
         described(_lib.SSD_F32, (b, H, P, N)), dims, 1, None)
     assert rc == _lib.SSD_ERR_SCRATCH, rc
     assert "workspace" in lib.ssd_status_string(rc).decode()
+
+
+def test_static_entry_point_inside_a_hip_graph(oracle):
+    # What the entry point is for: a caller that may not allocate, here HIP graph capture.  The call is captured once
+    # (its scratch is cleared by a kernel, not by a memset node) and replayed three times, with eager work and
+    # synchronisations between the replays and new input values each time; every replay must give the bits of an
+    # eager call on the same values.
+    import ssd_amd as ops
+    d = oracle.make_inputs(2, b=1, L=8192, H=16)
+    B, x, dt, dA = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    init = _dev(d["initial_states"])
+    b, L, H, P = x.shape
+    N, C = B.shape[-1], dt.shape[2]
+    out = torch.empty((b, C, H, P, N), device="cuda")
+    fin = torch.empty((b, H, P, N), device="cuda")
+    x_live = x.clone()
+    print(f"[static.graph] x{tuple(x.shape)} chunks={C}", flush=True)
+    ops._fused_chunk_state_state_passing_fwd_static(B, x_live, dt, dA, out, fin, initial_states=init)   # set-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops._fused_chunk_state_state_passing_fwd_static(B, x_live, dt, dA, out, fin, initial_states=init)
+    for scale in (1.0, -0.5, 3.0):
+        x_live.copy_((x.float() * scale).to(x.dtype))
+        out.fill_(float("nan")); fin.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ops._fused_static_status() == 0
+        want_out, want_fin = ops._fused_chunk_state_state_passing_fwd(B, x_live, dt, dA, torch.float32, initial_states=init, _kernel=1)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_out) and torch.equal(fin, want_fin), f"replay with x * {scale}"
+    ref_out, _ = oracle.fused_ref(d["B"], (d["x"].float() * 3.0).to(d["x"].dtype), d["dt"], d["dA_cumsum"],
+                                  initial_states=d["initial_states"])
+    err = (out.cpu() - ref_out).abs()
+    assert int((err > 1e-3 + 2e-3 * ref_out.abs()).sum()) == 0, f"max abs err {float(err.max()):.3e}"
