@@ -722,10 +722,13 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     const int n_units = p.n_items >> 2;
     p.n_xcd = n_cu >= 32 ? n_cu / 32 : 1;
     if (p.n_xcd > chain::kMaxXcd) p.n_xcd = chain::kMaxXcd;
-    // LOCAL pays when an XCD has enough units of its own to keep its compute units on different chains (measured:
-    // 20 units per XCD 213 against 224 us; 5 per XCD 568 against 254 us) and the units spread evenly.
+    // LOCAL when the units spread evenly over the XCDs and each has a few of its own: producer and consumer of a passed
+    // state then share an L2 (no read-back from memory), and an XCD only fetches the B rows of its own units' groups
+    // (b=1 L=131072 H=128 G=8: 5.3 GB of HBM traffic instead of 6.5 GB for 4.7 GB algorithmic, 1.15 ms
+    // against 1.17 ms).  With one or
+    // two units per XCD most of its workgroups would sit in one chain.
     const int fullest = (n_units + p.n_xcd - 1) / p.n_xcd;
-    const bool local = mode == 1 || (mode == 0 && n_units >= 16 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
+    const bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
     // Chunks per item: as many as leave every workgroup a few items (the parked chunk states fill the register file:
     // one workgroup per compute unit).  p.n_seg > 0 forces a value.
     int r = p.n_seg > 0 ? p.n_seg : 4;
