@@ -1,0 +1,171 @@
+"""CPU model of the ticket / flag-chain protocol of csrc/ssd_chain.hip (the replacement of the reference's global
+barrier, kernels/fused_globalbar.py:130-137, and of its completion counters and throttle semaphore,
+kernels/fused_concurrent.py:81-84, 141, 205-208).
+
+The model keeps what the argument for the kernel rests on and nothing else: a ticket counter, chunk-major work items
+(ticket t -> chunks R (t / units) .., unit t % units), workgroups that work through their tickets in the order they
+drew them and draw one ticket per item (the second during the first chunk of the first item, the third during its
+second chunk), a flag per (unit, chunk) raised after the item's last state is stored, a bounded wait that gives up,
+reports and still raises its flag, and the cut of an item at a sequence start.  Workgroups are advanced one event at a
+time by an adversarial (seeded random) scheduler with a limit on how many may be resident, down to one -- the hardware
+promises nothing about residency.  Checked: every launch drains, every passed state equals the serial recurrence
+(ssd_state_passing.py:69-84 on scalars), no wait gives up when the limit is generous, and a limit of one poll is
+reported while the launch still drains."""
+import random
+
+import pytest
+
+
+class Launch:
+    def __init__(self, n_units, C, R, n_wg, resident, spin_limit, seed, boundaries=()):
+        self.n_units, self.C, self.R, self.n_wg, self.resident, self.spin_limit = n_units, C, R, n_wg, resident, spin_limit
+        self.rng = random.Random(seed)
+        self.n_super = (C + R - 1) // R
+        self.total = n_units * self.n_super
+        self.ticket = 0
+        self.error = 0
+        self.flag = [[0] * (C + 1) for _ in range(n_units)]
+        # per (unit, chunk): chunk state S and decay d (zero where a sequence starts)
+        self.S = [[self.rng.uniform(-1, 1) for _ in range(C)] for _ in range(n_units)]
+        self.d = [[0.0 if (u, c) in boundaries else self.rng.uniform(0.1, 0.9) for c in range(C)] for u in range(n_units)]
+        self.init = [self.rng.uniform(-1, 1) for _ in range(n_units)]
+        self.out = [[None] * (C + 1) for _ in range(n_units)]       # out[u][c] = state entering chunk c; [C] = final
+        self.events = 0
+
+    def draw(self):
+        t = self.ticket
+        self.ticket += 1
+        return t
+
+    def item(self, t):
+        k, u = divmod(t, self.n_units)
+        return u, k * self.R, min(self.C, (k + 1) * self.R)
+
+    def workgroup(self):
+        """One persistent workgroup as a generator: every `yield` is a point where the scheduler may switch."""
+        cur = self.draw()
+        if cur >= self.total:
+            return
+        u, c0, c1 = self.item(cur)
+        single = c1 - c0 == 1
+        nxt = self.draw() if single else None          # a first item of one chunk needs its successor at once
+        late = nxt is None
+        after = None
+        yield
+        while cur < self.total:
+            u, c0, c1 = self.item(cur)
+            n = c1 - c0
+            held = []
+            for r in range(n):                         # the chunks of the item: independent of every other chunk
+                if r == 0 or (late and r == 1):
+                    t_new = self.draw()
+                    if late and r == 0:
+                        nxt = t_new
+                    else:
+                        after = t_new
+                held.append(self.S[u][c0 + r])
+                yield
+            scale = [self.d[u][c0 + r] for r in range(n)]
+            jz = max([r for r in range(1, n) if scale[r] == 0.0], default=0)
+
+            def hand_on():
+                self.out[u][c0 + n] = held[n - 1]
+                yield                                  # the store is acknowledged ...
+                if c0 + n < self.C:
+                    self.flag[u][c0 + n] = 1           # ... before the flag goes up
+
+            if jz > 0:                                 # a sequence starts inside the item: the part behind it first
+                for r in range(jz + 1, n):
+                    held[r] += scale[r] * held[r - 1]
+                yield from hand_on()
+            use_prev = scale[0] != 0.0
+            if use_prev and c0 > 0:
+                polls = 0
+                while not self.flag[u][c0]:
+                    polls += 1
+                    if polls >= self.spin_limit:
+                        self.error |= 1
+                        break
+                    yield
+            if c0 == 0:
+                self.out[u][0] = self.init[u]
+            if use_prev:
+                prev = self.out[u][c0] if self.out[u][c0] is not None else float("nan")   # gave up: whatever is there
+                held[0] += scale[0] * prev
+            for r in range(1, jz if jz > 0 else n):
+                held[r] += scale[r] * held[r - 1]
+            if jz == 0:
+                yield from hand_on()
+            for r in range(n - 1):                     # the states inside the item
+                self.out[u][c0 + r + 1] = held[r]
+            yield
+            cur, nxt, after, late = nxt, after, None, False
+
+    def run(self):
+        waiting = [self.workgroup() for _ in range(self.n_wg)]      # dispatched in order, `resident` at a time
+        running = []
+        budget = 200 * (self.total + self.n_wg) * max(4, min(self.spin_limit, 64))
+        while waiting or running:
+            while waiting and len(running) < self.resident:
+                running.append(waiting.pop(0))
+            g = self.rng.choice(running)
+            try:
+                next(g)
+            except StopIteration:
+                running.remove(g)
+            self.events += 1
+            assert self.events < budget, "the launch does not drain"
+        return self
+
+    def reference(self):
+        want = []
+        for u in range(self.n_units):
+            s, row = self.init[u], [self.init[u]]
+            for c in range(self.C):
+                s = self.d[u][c] * s + self.S[u][c]
+                row.append(s)
+            want.append(row)
+        return want
+
+
+SHAPES = [(5, 32, 4, 32), (1, 16, 4, 8), (7, 9, 2, 16), (3, 5, 1, 8), (40, 8, 4, 16), (2, 1, 4, 4), (6, 3, 4, 64)]
+
+
+@pytest.mark.parametrize("resident", [1, 2, 3, 1000])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "units%d-C%d-R%d-wg%d" % s)
+def test_every_schedule_drains_and_matches_the_serial_recurrence(shape, resident):
+    n_units, C, R, n_wg = shape
+    for seed in range(12):
+        rng = random.Random(1000 + seed)
+        boundaries = {(rng.randrange(n_units), rng.randrange(C)) for _ in range((n_units * C) // 7)} if seed % 2 else set()
+        L = Launch(n_units, C, R, n_wg, resident, spin_limit=1 << 30, seed=seed, boundaries=boundaries).run()
+        assert L.error == 0
+        assert L.ticket >= L.total
+        want = L.reference()
+        for u in range(n_units):
+            for c in range(C + 1):
+                assert L.out[u][c] is not None, (u, c)
+                assert abs(L.out[u][c] - want[u][c]) <= 1e-12 * max(1.0, abs(want[u][c])), (u, c, seed)
+
+
+def test_an_item_only_ever_waits_for_a_smaller_ticket():
+    # the order argument itself: the item a ticket depends on has the ticket `units` below it
+    L = Launch(5, 32, 4, 32, 1000, 1 << 30, 0)
+    for t in range(L.total):
+        u, c0, _ = L.item(t)
+        if c0 > 0:
+            up, _, c1p = L.item(t - L.n_units)
+            assert up == u and c1p == c0
+
+
+@pytest.mark.parametrize("resident", [2, 1000])
+def test_a_wait_that_runs_out_is_reported_and_the_launch_still_drains(resident):
+    reported = 0
+    for seed in range(20):
+        L = Launch(3, 16, 1, 16, resident, spin_limit=1, seed=seed).run()
+        reported += L.error
+        for u in range(3):
+            assert L.flag[u][16] == 0 and all(L.flag[u][c] for c in range(1, 16))     # every flag was raised all the same
+    assert reported > 0
+    # and with one resident workgroup nothing ever waits: it meets its own finished items
+    assert Launch(3, 16, 1, 16, 1, spin_limit=1, seed=0).run().error == 0
