@@ -301,12 +301,6 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 
     // acc[it][jp][r]: dstate column 16*it + 4*kg + r of headdim row p0 + 2*i16 + jp
     f32x4 acc[NT][2];
-    auto zero_acc = [&]() {
-#pragma unroll
-        for (int it = 0; it < NT; ++it)
-#pragma unroll
-            for (int jp = 0; jp < 2; ++jp) acc[it][jp] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    };
 
     // ---- chunk states parked in registers, and the chain step of an item --------------------------------------
     // The accumulators hold a 16 x 16 block as (lane%16 = row, lane/16 = group of four columns); each block passes
@@ -533,7 +527,6 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     }
     Meta mnext = mcur;
     int t_new = 0;          // the ticket drawn during this item (wave 0, lane 0)
-    zero_acc();
     // One 32-token step s of the current item (weight slot ws): fc = x operands of this step, fn receives those of
     // the step after it (the next item's first step after the last one).  Vector-memory requests of a step, in
     // program order: the two x requests of step + 3 (iteration 0), this wave's B requests of step + 3 (after the
@@ -587,8 +580,10 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
                         blo[tn % 4], bhi[tn % 4]);
             }
-            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
-            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
+            // a chunk's first step starts its sums: the accumulators are not cleared, the MFMA takes zero instead
+            constexpr f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, s == 0 ? zero : acc[it][0], 0, 0, 0);
+            acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, s == 0 ? zero : acc[it][1], 0, 0, 0);
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l1, acc[it][1], 0, 0, 0);
             // next step's x operands, spread over the iterations after the first (their LDS reads, issued at the top
@@ -619,7 +614,6 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             step(std::integral_constant<int, 7>{}, ws, fB, fA);
         }
         park(cur, mcur);
-        zero_acc();
         if (second_late && cur.r == 0) t_nxt = __builtin_amdgcn_readfirstlane(tq[1]);     // drawn during this chunk
         if (!(cur.r + 1 < R && cur.c + 1 < C)) {
             // the item's last chunk: the chain step, then the tickets move up
