@@ -127,13 +127,13 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  * all compute units.  The reference does the same job with scratch tensors it allocates per call: two ticket
  * counters and a global barrier (kernels/fused_globalbar.py:130-137, 237-238), or per-(batch, head) completion
  * counters plus a throttle semaphore (kernels/fused_concurrent.py:81-84, 141, 205-208, 296-298).  Here work items
- * (four state tiles sharing B x one chunk) are drawn from a device-wide ticket counter in chunk-major order; an
- * item accumulates its chunk state from zero, then waits for the flag of the state entering its chunk, reads that
- * state back from `out`, adds exp(dA_chunk) [same sequence] times it, stores the result as the next passed state
- * and raises the next flag.  An item only waits for an item with a smaller ticket and tickets are drawn by running
- * workgroups only, so the chain makes progress whatever workgroups are resident.  The wait is bounded nevertheless
- * (spin_limit polls): a wave that gives up sets the error word of the workspace and still raises its own flag, so
- * the launch always drains; ssd_fused_workspace_status reports it.
+ * (four state tiles sharing B x up to four consecutive chunks) are drawn from a ticket counter in chunk-major order;
+ * an item accumulates its chunk states from zero, then waits for the flag of the state entering its first chunk,
+ * reads that state back from `out`, runs s <- exp(dA_chunk) [same sequence] s + chunk state over its chunks, stores
+ * the last state first and raises the next flag once that store is acknowledged.  An item only waits for an item with
+ * a smaller ticket and tickets are drawn by running workgroups only, so the chain makes progress whatever workgroups
+ * are resident.  The wait is bounded nevertheless (spin_limit polls): a wave that gives up sets the error word of the
+ * workspace and still raises its own flag, so the launch always drains; ssd_fused_workspace_status reports it.
  *
  * workspace: device memory, 4-byte aligned, at least ssd_fused_workspace_bytes(dims); the call clears what it uses
  * (a small fill launch, no memset node), so the memory may hold anything and may be reused by later calls on the
@@ -141,7 +141,11 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  * kernel: SSD_KERNEL_AUTO lets the library choose between this kernel and those of ssd_fused_chunk_state_passing_fwd
  * (which it runs when the shape, element types or a `states` output rule the chain kernel out: it needs bf16 x / B,
  * fp32 out / initial / final states, no `states`, dstate 64 or 128, chunk 128 or 256); SSD_KERNEL_CHAIN insists on it
- * and returns SSD_ERR_SCRATCH where it cannot run.  opts == NULL behaves as ssd_fused_chunk_state_passing_fwd.
+ * and returns SSD_ERR_SCRATCH where it cannot run; SSD_KERNEL_CHAIN_LOCAL / _GLOBAL also fix how passed states cross
+ * between compute units, which the library otherwise chooses from the number of units per XCD (LOCAL: one ticket
+ * counter per XCD over that XCD's share of the units, states exchanged through its L2; GLOBAL: one counter, states
+ * exchanged through memory with device-scope accesses).  The results do not depend on the choice beyond rounding.
+ * opts == NULL behaves as ssd_fused_chunk_state_passing_fwd.
  */
 typedef struct ssd_fused_opts {
     void *workspace;
