@@ -168,7 +168,9 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
 
 /*
  * Waits for `stream` and reads the error word of a workspace used by ssd_fused_chunk_state_passing_fwd_ws:
- * SSD_OK, or SSD_ERR_CHAIN_TIMEOUT when a wave of the last launch gave up waiting (the outputs are then unusable).
+ * SSD_OK, or SSD_ERR_CHAIN_TIMEOUT when a wave of the last launch of the chain kernel on this workspace gave up
+ * waiting (the outputs are then unusable).  A call that ran another kernel family (SSD_KERNEL_AUTO: see
+ * ssd_query_fused_plan) leaves the workspace alone; memory the chain kernel has never cleared reports SSD_OK.
  * No counterpart in the reference, whose spin loops are unbounded (kernels/fused_concurrent.py:11, 300).
  */
 int ssd_fused_workspace_status(const void *workspace, void *stream);
@@ -199,6 +201,28 @@ int ssd_fused_static_status(void *stream);
  * Pure host logic; launches nothing.
  */
 int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dims);
+
+/*
+ * Which kernel family a fused call on plain tensors of these sizes would run, and why: the library ranks its fused
+ * kernels by an estimate of their duration (a fit to measured times, per compute unit) and this call returns the
+ * ranking.  Assumed: bf16 x / B, fp32 dt / dA_cumsum / out / final_states, contiguous, no `states` output -- the
+ * arguments every family covers.  has_workspace != 0 asks about ssd_fused_chunk_state_passing_fwd_ws with a
+ * workspace of ssd_fused_workspace_bytes(dims) and SSD_KERNEL_AUTO, 0 about ssd_fused_chunk_state_passing_fwd.
+ * compute_units: of the device the call would run on; 0 = 256 (MI355X).  Pure host logic: touches no device and
+ * launches nothing, so it also answers on a machine without a GPU.  No counterpart in the reference, whose two fused
+ * wrappers each have one kernel (kernels/fused_globalbar.py:201-266, kernels/fused_concurrent.py:255-331).
+ * estimate_us[f] is 0 for a family that does not apply to the sizes.
+ */
+enum { SSD_FAMILY_GENERIC = 0, SSD_FAMILY_TOKEN_SPLIT = 1, SSD_FAMILY_FOUR_TILE = 2, SSD_FAMILY_PAIR = 3,
+       SSD_FAMILY_CHAIN = 4, SSD_FAMILY_COUNT = 5 };
+
+typedef struct ssd_fused_plan {
+    int32_t family;                         /* SSD_FAMILY_* the call would run */
+    int32_t chunks_per_item;                /* of the chain kernel when that is the family, else 0 */
+    float estimate_us[SSD_FAMILY_COUNT];    /* the model's estimate per family (chain: at its best chunks per item) */
+} ssd_fused_plan;
+
+int ssd_query_fused_plan(const ssd_dims *dims, int has_workspace, int compute_units, ssd_fused_plan *plan);
 
 /*
  * dt preparation and per-chunk cumulative sum, the producer of `dt` and `dA_cumsum` for the three calls above.

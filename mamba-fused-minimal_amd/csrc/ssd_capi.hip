@@ -1,6 +1,7 @@
 // extern "C" entry points of libssd_gfx950.so: argument validation, kernel-family selection, launch.
 #include "../../include/ssd_gfx950.h"
 #include "ssd_params.h"
+#include "ssd_cost.h"
 
 #include <stdlib.h>
 #include <string.h>
@@ -138,38 +139,54 @@ Params with_states_in_out(const Params &p)
     return q;
 }
 
+// What a call runs.  The values are those of ssd_fused_plan::family.
+enum Family { F_GENERIC = SSD_FAMILY_GENERIC, F_TOKEN_SPLIT = SSD_FAMILY_TOKEN_SPLIT, F_FOUR_TILE = SSD_FAMILY_FOUR_TILE,
+              F_PAIR = SSD_FAMILY_PAIR, F_CHAIN = SSD_FAMILY_CHAIN };
+struct Choice {
+    int family;
+    bool states_in_out;      // F_PAIR: `out` doubles as the place for the chunk states
+};
+
+// The kernel family of a call without a workspace.
+Choice choose(const Params &p, bool fused, int64_t n_cu)
+{
+    // Fused launch: with at least two state tiles per compute unit the four-tiles-per-workgroup kernel wins (B is
+    // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
+    // kernel, which puts four waves on every tile, has the shorter chunk.
+    const int tiles = p.batch * p.nheads * (p.headdim / 32);
+    const int forced = g_forced_split.load(std::memory_order_relaxed);      // one value for the whole choice
+    if (fused && (forced == 1 || (forced == 0 && tiles >= 2 * n_cu)) && ssd::quad_supported(p)) return {F_FOUR_TILE, false};
+    // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
+    // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
+    // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
+    if (fused && !p.states && forced == 0 && tiles < 2 * n_cu && (int64_t)tiles * p.C >= 32 * n_cu &&
+        p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p)))
+        return {F_PAIR, true};
+    // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
+    // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
+    // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
+    if (fused && p.states && (forced == 1 || (forced == 0 && (int64_t)tiles * p.C >= 32 * n_cu)) && pair_supported(p))
+        return {F_PAIR, false};
+    if (!fused && (forced == 1 || (forced == 0 && (int64_t)tiles * p.C >= 8 * n_cu)) && ssd::quad_chunk_state_supported(p))
+        return {F_FOUR_TILE, false};
+    return {ssd::mfma_supported(p) ? F_TOKEN_SPLIT : F_GENERIC, false};
+}
+
 int run(const Params &p_in, bool fused, void *stream)
 {
     int rc = check_device();
     if (rc) return rc;
     Params p = p_in;
     p.n_cu = compute_units();
-    const int64_t n_cu = p.n_cu > 0 ? p.n_cu : 256;
     hipStream_t s = (hipStream_t)stream;
+    const Choice c = choose(p, fused, p.n_cu > 0 ? p.n_cu : 256);
     hipError_t e;
-    // Fused launch: with at least two state tiles per compute unit the four-tiles-per-workgroup kernel wins (B is
-    // fetched once per four tiles and the state never leaves the accumulators); with fewer, the token-split
-    // kernel, which puts four waves on every tile, has the shorter chunk.
-    const int tiles = p.batch * p.nheads * (p.headdim / 32);
-    const int g_forced_split = ::g_forced_split.load(std::memory_order_relaxed);      // one value for the whole choice
-    if (fused && (g_forced_split == 1 || (g_forced_split == 0 && tiles >= 2 * n_cu)) && ssd::quad_supported(p))
-        e = ssd::launch_quad(p, s);
-    else if (fused && !p.states && g_forced_split == 0 && tiles < 2 * n_cu && (int64_t)tiles * p.C >= 32 * n_cu &&
-             p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p))) {
-        // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
-        // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
-        // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
-        e = launch_pair(with_states_in_out(p), s);
-    } else if (fused && p.states && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 32 * n_cu)) &&
-               pair_supported(p)) {
-        // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
-        // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
-        // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
-        e = launch_pair(p, s);
-    } else if (!fused && (g_forced_split == 1 || (g_forced_split == 0 && (int64_t)tiles * p.C >= 8 * n_cu)) &&
-             ssd::quad_chunk_state_supported(p))
-        e = ssd::launch_quad_chunk_state(p, s);
-    else e = ssd::mfma_supported(p) ? ssd::launch_mfma(p, fused, s) : ssd::launch_generic(p, fused, s);
+    switch (c.family) {
+        case F_FOUR_TILE: e = fused ? ssd::launch_quad(p, s) : ssd::launch_quad_chunk_state(p, s); break;
+        case F_PAIR: e = launch_pair(c.states_in_out ? with_states_in_out(p) : p, s); break;
+        case F_TOKEN_SPLIT: e = ssd::launch_mfma(p, fused, s); break;
+        default: e = ssd::launch_generic(p, fused, s); break;
+    }
     return (int)e;
 }
 
@@ -201,13 +218,39 @@ hipError_t scratch_pointer(int **ptr)
     return hipSuccess;
 }
 
-// Whether the ticket / flag-chain kernel is the better fused kernel for a problem it covers: it keeps every compute
-// unit busy whatever the number of state tiles, at the price of reading each passed state back once.
-bool chain_preferred(const Params &p)
+// The fused problem as the cost model sees it.
+ssd::cost::Problem problem_of(const Params &p, int n_cu)
 {
-    // it needs several items of four chunks per compute unit to pay for its start and its chain
-    const int64_t units = (int64_t)p.batch * p.nheads * (p.headdim / 32) / 4;
-    return p.C >= 16 && units * (p.C / 4) >= 3 * (int64_t)compute_units();
+    ssd::cost::Problem q;
+    q.units = (int64_t)p.batch * p.nheads * (p.headdim / 32) / 4;
+    q.chunks = p.C; q.chunk_size = p.Q; q.dstate = p.dstate;
+    q.n_cu = n_cu > 0 ? n_cu : 256;
+    return q;
+}
+
+// Estimate for the family `c` (what the call would run without a workspace); a family the model does not cover
+// counts as slower than anything.
+double estimate_us(const ssd::cost::Problem &q, const Choice &c)
+{
+    switch (c.family) {
+        case F_FOUR_TILE: return ssd::cost::four_tile_us(q);
+        case F_PAIR: return ssd::cost::pair_us(q);
+        case F_TOKEN_SPLIT: return ssd::cost::token_split_us(q);
+        default: return 1e30;
+    }
+}
+
+// Whether the ticket / flag-chain kernel is the better fused kernel for a problem it covers: it keeps every compute
+// unit busy whatever the number of state tiles, at the price of its start, of reading each passed state back once per
+// item and of a link per item.
+bool chain_preferred(const Params &p, int n_cu)
+{
+    const ssd::cost::Problem q = problem_of(p, n_cu);
+    double chain = 0.;
+    ssd::cost::chain_chunks_per_item(q, &chain);
+    // within the model's error the chain kernel gets the call: its time follows the amount of work, the others'
+    // depends on how their workgroups happen to fall on the compute units
+    return chain < 1.05 * estimate_us(q, choose(p, true, q.n_cu));
 }
 
 }  // namespace
@@ -298,7 +341,7 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
     if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
     const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
                          opts->workspace_bytes >= ssd_fused_workspace_bytes(dims);
-    if (have_ws && ssd::chain_supported(p) && (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p)))) {
+    if (have_ws && ssd::chain_supported(p) && (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
         rc = check_device();
         if (rc) return rc;
         p.ws = (int *)opts->workspace;
@@ -346,11 +389,14 @@ int ssd_fused_workspace_status(const void *workspace, void *stream)
     if (!workspace) return SSD_ERR_NULL;
     int rc = check_device();
     if (rc) return rc;
-    int word = 0;       // the error word sits behind the sixteen ticket counters
-    hipError_t e = hipMemcpyAsync(&word, (const int *)workspace + 16, sizeof(word), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    static_assert(ssd::kChainWsTagWord == ssd::kChainWsErrWord + 1, "read in one copy");
+    int word[2] = {0, 0};       // error word and tag, behind the sixteen ticket counters
+    hipError_t e = hipMemcpyAsync(word, (const int *)workspace + ssd::kChainWsErrWord, sizeof(word), hipMemcpyDeviceToHost,
+                                  (hipStream_t)stream);
     if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return (int)e;
-    return word ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
+    if (word[1] != ssd::kChainWsTag) return SSD_OK;      // the chain kernel has not run on this memory: nothing to report
+    return word[0] ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
 }
 
 int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
@@ -422,6 +468,45 @@ int ssd_query_path(const ssd_tensor *x, const ssd_tensor *B, const ssd_dims *dim
     int rc = fill_common(p, x, B, &f32, &f32, nullptr, nullptr, dims, 1);
     if (rc) return rc;
     return ssd::mfma_supported(p) ? 1 : 0;
+}
+
+int ssd_query_fused_plan(const ssd_dims *dims, int has_workspace, int compute_units, ssd_fused_plan *plan)
+{
+    if (!plan) return SSD_ERR_NULL;
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    if (compute_units < 0) return SSD_ERR_SHAPE;
+    // plain tensors of these sizes at a made-up, well-aligned address: only sizes, strides and types are looked at
+    const int64_t L = dims->seqlen, H = dims->nheads, P = dims->headdim, N = dims->dstate,
+                  G = dims->ngroups, Q = dims->chunk_size, C = dims->nchunks;
+    void *const somewhere = (void *)(uintptr_t)4096;
+    const ssd_tensor x = {somewhere, SSD_BF16, 0, {L * H * P, H * P, P, 1, 0}};
+    const ssd_tensor B = {somewhere, SSD_BF16, 0, {L * G * N, G * N, N, 1, 0}};
+    const ssd_tensor dt = {somewhere, SSD_F32, 0, {H * C * Q, C * Q, Q, 1, 0}};
+    const ssd_tensor out = {somewhere, SSD_F32, 0, {C * H * P * N, H * P * N, P * N, N, 1}};
+    const ssd_tensor fin = {somewhere, SSD_F32, 0, {H * P * N, P * N, N, 1, 0}};
+    Params p;
+    rc = fill_fused(p, &x, &B, &dt, &dt, nullptr, nullptr, nullptr, &out, &fin, dims, 1);
+    if (rc) return rc;
+    const int n_cu = compute_units > 0 ? compute_units : 256;
+    p.n_cu = n_cu;
+    memset(plan, 0, sizeof(*plan));
+    const ssd::cost::Problem q = problem_of(p, n_cu);
+    const Choice c = choose(p, true, n_cu);
+    if (ssd::mfma_supported(p)) plan->estimate_us[SSD_FAMILY_TOKEN_SPLIT] = (float)ssd::cost::token_split_us(q);
+    if (ssd::quad_supported(p)) plan->estimate_us[SSD_FAMILY_FOUR_TILE] = (float)ssd::cost::four_tile_us(q);
+    if (pair_supported(with_states_in_out(p))) plan->estimate_us[SSD_FAMILY_PAIR] = (float)ssd::cost::pair_us(q);
+    plan->family = c.family;
+    if (ssd::chain_supported(p)) {
+        double us = 0.;
+        const int r = ssd::cost::chain_chunks_per_item(q, &us);
+        plan->estimate_us[SSD_FAMILY_CHAIN] = (float)us;
+        if (has_workspace && g_forced_split.load(std::memory_order_relaxed) == 0 && us < 1.05 * estimate_us(q, c)) {
+            plan->family = SSD_FAMILY_CHAIN;
+            plan->chunks_per_item = r;
+        }
+    }
+    return SSD_OK;
 }
 
 int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *dt_out,

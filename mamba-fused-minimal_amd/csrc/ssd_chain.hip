@@ -33,6 +33,7 @@
 // operands, all requests three steps ahead -- across chunk and item boundaries: the ticket of the next item is known
 // while an item runs, so the first steps of the next chunk are always on their way when the current one ends.
 #include "ssd_tile.h"
+#include "ssd_cost.h"
 
 namespace ssd {
 
@@ -64,9 +65,10 @@ template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * N
 constexpr int kAuxDevice = 16;      // sc1
 constexpr int kMaxXcd = 16;
 
-// workspace: [0..15] ticket counters (one per XCD slot), [16] error word, [32..47] hardware id of the XCD that
-// took each slot (+1), flags from [kWsHeaderInts]
-constexpr int kWsHeaderInts = 64, kWsErr = 16, kWsOwner = 32;
+// workspace: [0..15] ticket counters (one per XCD slot), [16] error word, [17] a tag written with every clearing
+// (ssd_params.h: kChainWsTag), [32..47] hardware id of the XCD that took each slot (+1), flags from [kWsHeaderInts]
+constexpr int kWsHeaderInts = 64, kWsErr = kChainWsErrWord, kWsTag = kChainWsTagWord, kWsOwner = 32;
+constexpr int kWsTagValue = kChainWsTag;
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (4 or 8); R = chunks per work item (1, 2 or 4).
 // out, initial_states and final_states are fp32.
@@ -634,10 +636,11 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     }
 }
 
-// workspace cleared before every launch: ticket counter, error word and flags
+// workspace cleared before every launch: ticket counter, error word and flags; the tag says that the error word is
+// this kernel's (a workspace may hold anything before its first launch)
 __global__ void __launch_bounds__(256) clear_kernel(int *ws, int n)
 {
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = 0;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = i == kWsTag ? kWsTagValue : 0;
 }
 
 static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
@@ -723,10 +726,14 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     // two units per XCD most of its workgroups would sit in one chain.
     const int fullest = (n_units + p.n_xcd - 1) / p.n_xcd;
     const bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
-    // Chunks per item: as many as leave every workgroup a few items (the parked chunk states fill the register file:
-    // one workgroup per compute unit).  p.n_seg > 0 forces a value.
-    int r = p.n_seg > 0 ? p.n_seg : 4;
-    while (r > 1 && p.n_seg <= 0 && (int64_t)n_units * ((p.C + r - 1) / r) < 3 * (int64_t)n_cu) r >>= 1;
+    // Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units
+    // end up with too few or too unequal numbers of items that large.  p.n_seg > 0 forces a value.
+    int r = p.n_seg;
+    if (r <= 0) {
+        cost::Problem q;
+        q.units = n_units; q.chunks = p.C; q.chunk_size = p.Q; q.dstate = p.dstate; q.n_cu = n_cu > 0 ? n_cu : 256;
+        r = cost::chain_chunks_per_item(q, nullptr);
+    }
     const int64_t total = (int64_t)n_units * ((p.C + r - 1) / r);
     const int n_wg = (int)(total < n_cu ? total : n_cu);
     if (p.seq) return local ? launch_chain_t<true, true>(p, r, n_wg, s) : launch_chain_t<true, false>(p, r, n_wg, s);

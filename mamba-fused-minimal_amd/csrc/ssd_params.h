@@ -164,6 +164,9 @@ int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup o
 hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
 bool chain_supported(const Params &p);
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
+// Words of a chain workspace that the host reads back: the error word, and behind it a tag that every launch of the
+// chain kernel writes when it clears the workspace -- without it the error word is whatever the memory held.
+constexpr int kChainWsErrWord = 16, kChainWsTagWord = 17, kChainWsTag = 0x53534443;
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

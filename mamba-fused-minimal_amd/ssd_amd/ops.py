@@ -202,6 +202,20 @@ def _fused_workspace_status(workspace):
         return int(_lib.load().ssd_fused_workspace_status(ctypes.c_void_p(workspace.data_ptr()), _stream(workspace)))
 
 
+def fused_plan(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, workspace=True, compute_units=0):
+    """Which kernel family the fused call would run on plain bf16 / fp32 tensors of these sizes and the library's
+    estimate of every family's duration (no counterpart in the reference, whose fused wrappers have one kernel each:
+    kernels/fused_globalbar.py:201-266, kernels/fused_concurrent.py:255-331).  Host logic only: needs no GPU.
+    Returns {"family": name, "chunks_per_item": R or 0, "estimate_us": {name: microseconds or None}}."""
+    nchunks = (seqlen + chunk_size - 1) // chunk_size
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    plan = _lib.SsdFusedPlan()
+    _lib.check(_lib.load().ssd_query_fused_plan(dims, 1 if workspace else 0, int(compute_units), ctypes.byref(plan)),
+               "ssd_query_fused_plan")
+    return {"family": _lib.SSD_FAMILIES[plan.family], "chunks_per_item": int(plan.chunks_per_item),
+            "estimate_us": {n: (float(v) if v > 0 else None) for n, v in zip(_lib.SSD_FAMILIES, plan.estimate_us)}}
+
+
 def _fused_chunk_state_state_passing_fwd_globalbar(B, x, dt, dA_cumsum, out_dtype, initial_states=None,
                                                    seq_idx=None, states=None, states_in_fp32=True):
     """Drop-in for kernels/fused_globalbar.py:201 (same signature and returns)."""

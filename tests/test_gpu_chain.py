@@ -97,6 +97,22 @@ def test_chain_kernel_at_benchmark_configs(ops, oracle, cfg):
     _chain_case(ops, oracle, d, 1, 0, f"chain.cfg{cfg}")
 
 
+@pytest.mark.parametrize("kw, family, r", [
+    (dict(b=1, L=8192, H=80), "chain", 2),        # 40 units x 32 chunks: two chunks per item fill the device evenly
+    (dict(b=8, L=2048, H=80), "chain", 2),        # 8 chunks only, 320 units
+    (dict(b=3, L=4096, H=80), "chain", 4),
+    (dict(b=4, L=2048, H=80), "four_tile", 0),    # 160 units x 8 chunks: one workgroup per unit is faster
+    (dict(b=2, L=2048, H=80), "token_split", 0),  # 80 units x 8 chunks
+], ids=["b1-L8192", "b8-L2048", "b3-L4096", "b4-L2048", "b2-L2048"])
+def test_shapes_between_the_benchmark_configs_on_the_kernel_the_library_picks(ops, oracle, kw, family, r):
+    # the choice is made from an estimate of each family's duration; whatever it picks has to be right
+    d = oracle.make_inputs(2, **kw)
+    cfg = d["cfg"]
+    plan = ops.fused_plan(cfg["b"], cfg["L"], cfg["H"], cfg["P"], cfg["N"], cfg["G"], cfg["Q"])
+    assert (plan["family"], plan["chunks_per_item"]) == (family, r), plan
+    _chain_case(ops, oracle, d, 0, 0, "auto." + "-".join(f"{k}{v}" for k, v in kw.items()))
+
+
 def test_chain_matches_the_other_fused_kernels(ops, oracle):
     # same inputs through the chain kernel and through the kernel the workspace-less entry point picks
     d = oracle.make_inputs(2, b=2, L=4096, H=16)
