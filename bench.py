@@ -166,6 +166,13 @@ def main():
     def cumsum(i):
         return ssd_amd._chunk_cumsum_fwd(raw[i % nsets], A_dev, cfg["Q"], dt_bias=bias_dev, dt_softplus=True)
 
+    # producer + path in one call (two launches: the producer's clears the chain kernel's workspace on its way)
+    def prep_fused(i):
+        s = sets[i % nsets]
+        return ssd_amd._fused_cumsum_chunk_state_state_passing_fwd(
+            s["B"], s["x"], raw[i % nsets], A_dev, cfg["Q"], torch.float32, dt_bias=bias_dev, dt_softplus=True,
+            initial_states=s["initial_states"], seq_idx=s["seq_idx"])
+
     # the consumer of the passed states (state half of the chunk scan), fp32 y, on the states of the timed launches
     C_dev = [mv(d["C"]).clone() for _ in range(nsets)]
     prev_states = [fused(i)[0] for i in range(nsets)]
@@ -178,6 +185,7 @@ def main():
 
     _, bf16_ev = timed(fused_bf16, max(5, args.steps // 4), 3)
     _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
+    _, prep_ev = timed(prep_fused, max(5, args.steps // 4), 3)
     _, scan_ev = timed(scan_states, max(5, args.steps // 4), 3)
     del prev_states, y_bufs
 
@@ -238,6 +246,7 @@ def main():
         "unfused_us": round(unf_ev * 1e6, 2),
         "fused_bf16_out_us": round(bf16_ev * 1e6, 2),
         "chunk_cumsum_us": round(cs_ev * 1e6, 2),
+        "fused_with_dt_preparation_us": round(prep_ev * 1e6, 2),
         "chunk_scan_states_us": round(scan_ev * 1e6, 2),
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,

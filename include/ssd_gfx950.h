@@ -253,6 +253,21 @@ int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tens
                                              float dt_min, float dt_max, int clamp, void *stream);
 
 /*
+ * The same with a workspace (ssd_fused_opts as in ssd_fused_chunk_state_passing_fwd_ws), which opens the ticket /
+ * flag-chain kernel to this call as well.  Still two launches: where that kernel runs, the producer's launch clears
+ * its workspace on the way, so the fill launch of ssd_fused_chunk_state_passing_fwd_ws is not needed.  Without a
+ * usable workspace it behaves as ssd_fused_cumsum_chunk_state_passing_fwd.  No counterpart in the reference beyond
+ * the two calls it composes (kernels/ssd_chunk_state.py:176-199, kernels/fused_concurrent.py:255-331).
+ */
+int ssd_fused_cumsum_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
+                                                const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *seq_idx,
+                                                const ssd_tensor *initial_states, const ssd_tensor *dt_out,
+                                                const ssd_tensor *dA_cumsum, const ssd_tensor *out,
+                                                const ssd_tensor *final_states, const ssd_dims *dims, int dt_softplus,
+                                                float dt_min, float dt_max, int clamp, const ssd_fused_opts *opts,
+                                                void *stream);
+
+/*
  * The consumer of the passed states: the state-dependent half of the chunk scan.  Replaces that part of
  * _chunk_scan_fwd_kernel (kernels/ssd_chunk_scan.py:94-117; wrapper _chunk_scan_fwd, :172-224):
  *   y[b,cQ+m,h,p] = scale_m * sum_n C[b,cQ+m,h/(H/G),n] * prev_states[b,c,h,p,n],

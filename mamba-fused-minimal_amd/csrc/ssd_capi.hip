@@ -253,6 +253,60 @@ bool chain_preferred(const Params &p, int n_cu)
     return chain < 1.05 * estimate_us(q, choose(p, true, q.n_cu));
 }
 
+// Whether a fused call runs on the ticket / flag-chain kernel: a usable workspace came with it and that kernel is
+// asked for or estimated to be the faster one.  Returns a status (a kernel forced where it cannot run).
+int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *opts, bool *use)
+{
+    *use = false;
+    const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
+    if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
+    const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
+                         opts->workspace_bytes >= ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+    if (have_ws && ssd::chain_supported(p) &&
+        (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
+        *use = true;
+        return check_device();
+    }
+    return kernel != SSD_KERNEL_AUTO ? SSD_ERR_SCRATCH : SSD_OK;     // forced, but no workspace or not a shape it covers
+}
+
+int run_chain(Params &p, const ssd_fused_opts *opts, void *stream)
+{
+    p.ws = (int *)opts->workspace;
+    p.spin_limit = opts->spin_limit;
+    p.n_seg = opts->chunks_per_item == 1 || opts->chunks_per_item == 2 || opts->chunks_per_item == 4 ? opts->chunks_per_item : 0;
+    return (int)ssd::launch_chain(p, compute_units(),
+                                  opts->kernel == SSD_KERNEL_CHAIN_LOCAL ? 1 : opts->kernel == SSD_KERNEL_CHAIN_GLOBAL ? 2 : 0,
+                                  (hipStream_t)stream);
+}
+
+// Arguments of the dt preparation as its kernel takes them.
+int fill_cumsum(ssd::CumsumParams &p, const ssd_tensor *dt, const ssd_tensor *A, const ssd_tensor *dt_bias,
+                const ssd_tensor *dt_out, const ssd_tensor *dA_cumsum, int32_t batch, int32_t seqlen, int32_t nheads,
+                int32_t chunk_size, int dt_softplus, float dt_min, float dt_max)
+{
+    if (!present(dt) || !present(A) || !present(dt_out) || !present(dA_cumsum)) return SSD_ERR_NULL;
+    if (batch <= 0 || seqlen <= 0 || nheads <= 0 || chunk_size <= 0) return SSD_ERR_SHAPE;
+    if (!dtype_ok(dt->dtype) || !dtype_ok(A->dtype) || dt_out->dtype != SSD_F32 || dA_cumsum->dtype != SSD_F32)
+        return SSD_ERR_DTYPE;
+    memset(&p, 0, sizeof(p));
+    p.dt = dt->data; p.dt_type = dt->dtype;
+    p.sdt_b = dt->stride[0]; p.sdt_l = dt->stride[1]; p.sdt_h = dt->stride[2];
+    p.A = A->data; p.A_type = A->dtype; p.sA = A->stride[0];
+    if (present(dt_bias)) {
+        if (!dtype_ok(dt_bias->dtype)) return SSD_ERR_DTYPE;
+        p.dt_bias = dt_bias->data; p.dt_bias_type = dt_bias->dtype; p.sbias = dt_bias->stride[0];
+    }
+    p.dt_out = (float *)dt_out->data;
+    p.so_b = dt_out->stride[0]; p.so_h = dt_out->stride[1]; p.so_c = dt_out->stride[2]; p.so_k = dt_out->stride[3];
+    p.dacs = (float *)dA_cumsum->data;
+    p.sa_b = dA_cumsum->stride[0]; p.sa_h = dA_cumsum->stride[1]; p.sa_c = dA_cumsum->stride[2]; p.sa_k = dA_cumsum->stride[3];
+    p.batch = batch; p.seqlen = seqlen; p.nheads = nheads; p.Q = chunk_size;
+    p.C = (seqlen + chunk_size - 1) / chunk_size;
+    p.softplus = dt_softplus ? 1 : 0; p.dt_min = dt_min; p.dt_max = dt_max;
+    return ssd::chunk_cumsum_supported(p) ? SSD_OK : SSD_ERR_SHAPE;
+}
+
 }  // namespace
 
 extern "C" {
@@ -337,21 +391,10 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
     Params p;
     int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, states, out, final_states, dims, clamp);
     if (rc) return rc;
-    const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
-    if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
-    const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
-                         opts->workspace_bytes >= ssd_fused_workspace_bytes(dims);
-    if (have_ws && ssd::chain_supported(p) && (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
-        rc = check_device();
-        if (rc) return rc;
-        p.ws = (int *)opts->workspace;
-        p.spin_limit = opts->spin_limit;
-        p.n_seg = opts->chunks_per_item == 1 || opts->chunks_per_item == 2 || opts->chunks_per_item == 4 ? opts->chunks_per_item : 0;
-        return (int)ssd::launch_chain(p, compute_units(), kernel == SSD_KERNEL_CHAIN_LOCAL ? 1 : kernel == SSD_KERNEL_CHAIN_GLOBAL ? 2 : 0,
-                                      (hipStream_t)stream);
-    }
-    if (kernel != SSD_KERNEL_AUTO) return SSD_ERR_SCRATCH;     // forced, but no workspace or not a shape it covers
-    return run(p, true, stream);
+    bool chain = false;
+    rc = chain_decision(p, dims, opts, &chain);
+    if (rc) return rc;
+    return chain ? run_chain(p, opts, stream) : run(p, true, stream);
 }
 
 int ssd_fused_chunk_state_passing_fwd_static(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
@@ -406,21 +449,44 @@ int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tens
                                              const ssd_tensor *final_states, const ssd_dims *dims, int dt_softplus,
                                              float dt_min, float dt_max, int clamp, void *stream)
 {
-    if (!present(dt_raw) || !present(A)) return SSD_ERR_NULL;
-    if (!dtype_ok(dt_raw->dtype) || !dtype_ok(A->dtype)) return SSD_ERR_DTYPE;
-    if (present(dt_bias) && !dtype_ok(dt_bias->dtype)) return SSD_ERR_DTYPE;
+    return ssd_fused_cumsum_chunk_state_passing_fwd_ws(x, B, dt_raw, A, dt_bias, seq_idx, initial_states, dt_out, dA_cumsum, out,
+                                                       final_states, dims, dt_softplus, dt_min, dt_max, clamp, nullptr, stream);
+}
+
+int ssd_fused_cumsum_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
+                                                const ssd_tensor *A, const ssd_tensor *dt_bias, const ssd_tensor *seq_idx,
+                                                const ssd_tensor *initial_states, const ssd_tensor *dt_out,
+                                                const ssd_tensor *dA_cumsum, const ssd_tensor *out,
+                                                const ssd_tensor *final_states, const ssd_dims *dims, int dt_softplus,
+                                                float dt_min, float dt_max, int clamp, const ssd_fused_opts *opts,
+                                                void *stream)
+{
     Params p;
     int rc = fill_fused(p, x, B, dt_out, dA_cumsum, seq_idx, initial_states, nullptr, out, final_states, dims, clamp);
     if (rc) return rc;
-    // Two launches on the caller's stream.  A variant of the fused kernel that computes dt / dA_cumsum per chunk
-    // itself was built and measured: each of its workgroups walks two heads through the whole sequence and has to
-    // gather their two columns out of the token-major dt rows (a request per token and wave), which cost more
-    // (270 against 240 microseconds for both stages at batch 4 x 8192 tokens x 80 heads) than the producer's
-    // transposing pass and the read-back of its 21 MB.
-    rc = ssd_chunk_cumsum_fwd(dt_raw, A, dt_bias, dt_out, dA_cumsum, dims->batch, dims->seqlen, dims->nheads, dims->chunk_size,
-                              dt_softplus, dt_min, dt_max, stream);
+    ssd::CumsumParams cp;
+    rc = fill_cumsum(cp, dt_raw, A, dt_bias, dt_out, dA_cumsum, dims->batch, dims->seqlen, dims->nheads, dims->chunk_size,
+                     dt_softplus, dt_min, dt_max);
     if (rc) return rc;
-    return run(p, true, stream);
+    bool chain = false;
+    rc = chain_decision(p, dims, opts, &chain);
+    if (rc) return rc;
+    rc = check_device();
+    if (rc) return rc;
+    // Two launches on the caller's stream: the producer, which also clears the chain kernel's workspace on its way
+    // when that kernel follows, and the fused kernel.  Computing dt / dA_cumsum inside the fused kernels was built and
+    // measured for both of them and lost both times (batch 4 x 8192 tokens x 80 heads: 270 against 240 microseconds in
+    // the four-tile kernel, 232 against 197 in the chain kernel): their workgroups take two heads each and have to
+    // gather those two columns out of the token-major dt rows, a cache line per token, where the producer reads the
+    // rows whole.
+    if (chain) {
+        cp.clear = (int *)opts->workspace;
+        cp.n_clear = (int)(ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks) / sizeof(int));
+        p.ws_cleared = 1;
+    }
+    const hipError_t e = ssd::launch_chunk_cumsum(cp, (hipStream_t)stream);
+    if (e != hipSuccess) return (int)e;
+    return chain ? run_chain(p, opts, stream) : run(p, true, stream);
 }
 
 int ssd_state_passing_fwd(const ssd_tensor *states, const ssd_tensor *dA_chunk, const ssd_tensor *initial_states,
@@ -513,28 +579,10 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
                          const ssd_tensor *dA_cumsum, int32_t batch, int32_t seqlen, int32_t nheads, int32_t chunk_size,
                          int dt_softplus, float dt_min, float dt_max, void *stream)
 {
-    if (!present(dt) || !present(A) || !present(dt_out) || !present(dA_cumsum)) return SSD_ERR_NULL;
-    if (batch <= 0 || seqlen <= 0 || nheads <= 0 || chunk_size <= 0) return SSD_ERR_SHAPE;
-    if (!dtype_ok(dt->dtype) || !dtype_ok(A->dtype) || dt_out->dtype != SSD_F32 || dA_cumsum->dtype != SSD_F32)
-        return SSD_ERR_DTYPE;
     ssd::CumsumParams p;
-    memset(&p, 0, sizeof(p));
-    p.dt = dt->data; p.dt_type = dt->dtype;
-    p.sdt_b = dt->stride[0]; p.sdt_l = dt->stride[1]; p.sdt_h = dt->stride[2];
-    p.A = A->data; p.A_type = A->dtype; p.sA = A->stride[0];
-    if (present(dt_bias)) {
-        if (!dtype_ok(dt_bias->dtype)) return SSD_ERR_DTYPE;
-        p.dt_bias = dt_bias->data; p.dt_bias_type = dt_bias->dtype; p.sbias = dt_bias->stride[0];
-    }
-    p.dt_out = (float *)dt_out->data;
-    p.so_b = dt_out->stride[0]; p.so_h = dt_out->stride[1]; p.so_c = dt_out->stride[2]; p.so_k = dt_out->stride[3];
-    p.dacs = (float *)dA_cumsum->data;
-    p.sa_b = dA_cumsum->stride[0]; p.sa_h = dA_cumsum->stride[1]; p.sa_c = dA_cumsum->stride[2]; p.sa_k = dA_cumsum->stride[3];
-    p.batch = batch; p.seqlen = seqlen; p.nheads = nheads; p.Q = chunk_size;
-    p.C = (seqlen + chunk_size - 1) / chunk_size;
-    p.softplus = dt_softplus ? 1 : 0; p.dt_min = dt_min; p.dt_max = dt_max;
-    if (!ssd::chunk_cumsum_supported(p)) return SSD_ERR_SHAPE;
-    int rc = check_device();
+    int rc = fill_cumsum(p, dt, A, dt_bias, dt_out, dA_cumsum, batch, seqlen, nheads, chunk_size, dt_softplus, dt_min, dt_max);
+    if (rc) return rc;
+    rc = check_device();
     if (rc) return rc;
     return (int)ssd::launch_chunk_cumsum(p, (hipStream_t)stream);
 }

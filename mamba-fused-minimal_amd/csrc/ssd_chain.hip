@@ -640,7 +640,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 // this kernel's (a workspace may hold anything before its first launch)
 __global__ void __launch_bounds__(256) clear_kernel(int *ws, int n)
 {
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = i == kWsTag ? kWsTagValue : 0;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = chain_workspace_clear(i);
 }
 
 static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
@@ -710,10 +710,13 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     if (p.n_items <= 0 || p.C <= 0) return hipSuccess;
     if (p.spin_limit <= 0) p.spin_limit = 1 << 22;
     const int64_t n_ws = chain::kWsHeaderInts + (int64_t)p.n_items * p.C;
-    hipLaunchKernelGGL(chain::clear_kernel, dim3((unsigned)((n_ws + 255) / 256 < 1024 ? (n_ws + 255) / 256 : 1024)), dim3(256), 0, s,
-                       p.ws, (int)n_ws);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!p.ws_cleared) {
+        hipLaunchKernelGGL(chain::clear_kernel, dim3((unsigned)((n_ws + 255) / 256 < 1024 ? (n_ws + 255) / 256 : 1024)), dim3(256), 0, s,
+                           p.ws, (int)n_ws);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     // An XCD is 32 compute units on this part.  Units are dealt to the XCDs in contiguous ranges; LOCAL pays when
     // the fullest XCD holds at most an eighth more than its fair share of them.
     const int n_units = p.n_items >> 2;

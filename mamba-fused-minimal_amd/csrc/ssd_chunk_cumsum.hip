@@ -30,6 +30,11 @@ __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
     const int b = blockIdx.z, c = blockIdx.y, h0 = blockIdx.x * kHeadTile;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lim = min(Q, p.seqlen - c * Q);
+    if (p.clear) {
+        // on the way: the workspace of the chain kernel that this launch is in front of
+        const int n_wg = gridDim.x * gridDim.y * gridDim.z, wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        for (int i = wg * 256 + tid; i < p.n_clear; i += n_wg * 256) p.clear[i] = chain_workspace_clear(i);
+    }
 
     auto activate = [&](float d) {
         if (p.softplus && d <= 20.f) {

@@ -39,6 +39,7 @@ struct Params {
     int spin_limit;       // polls after which a wave of that kernel stops waiting for a flag
     int n_xcd;            // XCDs (L2 caches) the units of that kernel are dealt to
     int n_cu;             // compute units of the device (0: not known, the launchers then assume 256 in 8 XCDs)
+    int ws_cleared;       // the launch in front of that kernel has cleared `ws` already (chain_workspace_clear below)
 };
 
 // State passing on a flattened state axis.
@@ -73,6 +74,8 @@ struct CumsumParams {
     int dt_type, A_type, dt_bias_type;
     int softplus;
     float dt_min, dt_max;
+    int *clear;            // a chain workspace to clear on the way (the kernel behind this one is the chain kernel), or null
+    int n_clear;           // ints of it
 };
 
 // State-consuming half of the chunk scan: y = scale * (C . prev_states).
@@ -164,9 +167,14 @@ int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup o
 hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
 bool chain_supported(const Params &p);
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
+
 // Words of a chain workspace that the host reads back: the error word, and behind it a tag that every launch of the
 // chain kernel writes when it clears the workspace -- without it the error word is whatever the memory held.
 constexpr int kChainWsErrWord = 16, kChainWsTagWord = 17, kChainWsTag = 0x53534443;
+// The value a cleared chain workspace holds at int i: zero, except for the tag.  Any kernel that runs in front of the
+// chain kernel on the same stream may do the clearing (the stand-alone producer of dt / dA_cumsum does when both are
+// launched by one call); Params::ws_cleared then keeps the chain kernel's own fill launch away.
+__host__ __device__ constexpr int chain_workspace_clear(int i) { return i == kChainWsTagWord ? kChainWsTag : 0; }
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

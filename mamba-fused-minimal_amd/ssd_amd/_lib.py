@@ -15,7 +15,7 @@ _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
            "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes",
            "ssd_fused_workspace_status", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
-           "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_query_path", "ssd_query_fused_plan", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
+           "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd_ws", "ssd_query_path", "ssd_query_fused_plan", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
 class SsdTensor(ctypes.Structure):
@@ -76,6 +76,8 @@ def load():
     lib.ssd_fused_static_status.argtypes = [vp]
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.restype = ctypes.c_int
     lib.ssd_fused_cumsum_chunk_state_passing_fwd.argtypes = [T] * 11 + [D, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, vp]
+    lib.ssd_fused_cumsum_chunk_state_passing_fwd_ws.restype = ctypes.c_int
+    lib.ssd_fused_cumsum_chunk_state_passing_fwd_ws.argtypes = [T] * 11 + [D, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.POINTER(SsdFusedOpts), vp]
     lib.ssd_query_path.restype = ctypes.c_int
     lib.ssd_query_path.argtypes = [T, T, D]
     lib.ssd_query_fused_plan.restype = ctypes.c_int

@@ -254,10 +254,14 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
 
 def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dtype, dt_bias=None, dt_softplus=False,
                                                 dt_limit=(0.0, float("inf")), initial_states=None, seq_idx=None,
-                                                _clamp=True):
+                                                _clamp=True, _kernel=0, _chunks_per_item=0, _workspace=None):
     """``_chunk_cumsum_fwd`` followed by ``_fused_chunk_state_state_passing_fwd`` in one call (the first three stages of
     the reference's main.py:78-100): dt is the raw (batch, seqlen, nheads) tensor.  Returns
-    (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32, dA_cumsum, dt_out (b,H,C,Q) fp32)."""
+    (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32, dA_cumsum, dt_out (b,H,C,Q) fp32).
+
+    Two launches; where the library runs its ticket / flag-chain kernel, the first one clears that kernel's workspace
+    on its way.  ``_kernel``, ``_chunks_per_item`` and ``_workspace`` are the hooks of
+    ``_fused_chunk_state_state_passing_fwd``."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, ngroups, dstate = B.shape
     assert nheads % ngroups == 0
@@ -286,12 +290,16 @@ def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dty
     final_states = torch.empty((batch, nheads, headdim, dstate), device=x.device, dtype=torch.float32)
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
     T = _lib.tensor_arg
+    lib = _lib.load()
+    if _workspace is None:
+        _workspace = torch.empty(((int(lib.ssd_fused_workspace_bytes(dims)) + 3) // 4,), device=x.device, dtype=torch.int32)
+    opts = _lib.SsdFusedOpts(_workspace.data_ptr(), _workspace.numel() * 4, 0, int(_kernel), int(_chunks_per_item), 0)
     with torch.cuda.device(x.device):
-        rc = _lib.load().ssd_fused_cumsum_chunk_state_passing_fwd(
+        rc = lib.ssd_fused_cumsum_chunk_state_passing_fwd_ws(
             T(x), T(B), T(dt), T(A), T(dt_bias), T(seq_idx), T(initial_states), T(dt_out), T(dA_cumsum), T(out),
             T(final_states), dims, int(bool(dt_softplus)), float(dt_limit[0]), float(dt_limit[1]), 1 if _clamp else 0,
-            _stream(x))
-    _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd")
+            ctypes.byref(opts), _stream(x))
+    _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd_ws")
     return out, final_states, dA_cumsum, dt_out
 
 

@@ -113,6 +113,35 @@ def test_shapes_between_the_benchmark_configs_on_the_kernel_the_library_picks(op
     _chain_case(ops, oracle, d, 0, 0, "auto." + "-".join(f"{k}{v}" for k, v in kw.items()))
 
 
+@pytest.mark.parametrize("kernel", [0, LOCAL, GLOBAL], ids=["auto", "local", "global"])
+@pytest.mark.parametrize("kw", [dict(b=2, L=2048, H=8, init=True), dict(L=2000, H=8, nseq=5, init=True),
+                                dict(Q=128, L=1408, N=64, H=8)], ids=["base", "ragged-seq", "q128-n64"])
+def test_dt_preparation_and_chain_kernel_in_one_call(ops, oracle, kw, kernel):
+    # kernels/ssd_chunk_state.py:176-199 followed by the fused call, as one call with a workspace: the producer's launch
+    # clears the chain kernel's workspace (garbage here) on its way; same bits as the two calls made separately
+    d = oracle.make_inputs(2, **kw)
+    Q = d["cfg"]["Q"]
+    raw, A, bias, seq, init = d["dt_raw"], d["A"], d["dt_bias"], d["seq_idx"], d["initial_states"]
+    want_da, want_dt = oracle.chunk_cumsum_ref(raw, A, Q, dt_bias=bias, dt_softplus=True)
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], want_dt, want_da, initial_states=init, seq_idx=seq)
+    for rep in range(2):                                   # the second call finds the workspace as the first left it
+        ws = torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda") if rep == 0 else ws
+        out, fin, dA, dt = ops._fused_cumsum_chunk_state_state_passing_fwd(
+            _dev(d["B"]), _dev(d["x"]), _dev(raw), _dev(A), Q, torch.float32, dt_bias=_dev(bias), dt_softplus=True,
+            initial_states=_dev(init), seq_idx=_dev(seq), _kernel=kernel, _workspace=ws)
+        assert ops._fused_workspace_status(ws) == 0
+        for what, got, want, rtol, atol in (("dt", dt, want_dt, 2e-6, 1e-9), ("dA_cumsum", dA, want_da, 1e-5, 1e-6),
+                                            ("out", out, want_out, RTOL, ATOL), ("final", fin, want_fin, RTOL, ATOL)):
+            bad, worst = _mismatches(got, want, rtol, atol)
+            assert bad == 0, f"prep+chain.{what}: {bad} mismatches, max abs err {worst:.3e}"
+        dA2, dt2 = ops._chunk_cumsum_fwd(_dev(raw), _dev(A), Q, dt_bias=_dev(bias), dt_softplus=True)
+        out2, fin2 = ops._fused_chunk_state_state_passing_fwd(_dev(d["B"]), _dev(d["x"]), dt2, dA2, torch.float32,
+                                                              initial_states=_dev(init), seq_idx=_dev(seq), _kernel=kernel,
+                                                              _workspace=torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda"))
+        torch.cuda.synchronize()
+        assert torch.equal(dt2, dt) and torch.equal(dA2, dA) and torch.equal(out2, out) and torch.equal(fin2, fin)
+
+
 def test_chain_matches_the_other_fused_kernels(ops, oracle):
     # same inputs through the chain kernel and through the kernel the workspace-less entry point picks
     d = oracle.make_inputs(2, b=2, L=4096, H=16)
