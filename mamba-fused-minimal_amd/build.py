@@ -17,7 +17,10 @@ FLAGS = [
     # keep the compiler from forming packed-fp32 VALU instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
+    # one remark block per kernel with its registers, spills and scratch: collected into build/resource_usage.json
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+USAGE = os.path.join(OBJ_DIR, "resource_usage.json")
 
 
 def hipcc():
@@ -34,6 +37,28 @@ def _run(cmd):
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + out)
     return out
+
+
+def _resource_usage(text):
+    """Splits a compiler log into ({kernel: {field: value}}, the log without the resource-usage remarks)."""
+    import re
+    usage, rest, current, skip = {}, [], None, 0
+    for line in text.splitlines():
+        m = re.search(r"remark:\s+(.*?)\s+\[-Rpass-analysis=kernel-resource-usage\]", line)
+        if m:
+            key, _, value = m.group(1).partition(": ")
+            if key == "Function Name":
+                current = usage.setdefault(value.strip(), {})
+            elif current is not None:
+                value = value.strip()
+                current[key.strip()] = int(value) if value.lstrip("-").isdigit() else value
+            skip = 2                      # the source line and the caret that follow a remark
+        elif skip and (line.lstrip().startswith("|") or re.match(r"\s*\d+ \|", line)):
+            skip -= 1
+        else:
+            skip = 0
+            rest.append(line)
+    return usage, "\n".join(rest)
 
 
 def build_library(verbose=False, extra_flags=(), jobs=None):
@@ -53,12 +78,16 @@ def build_library(verbose=False, extra_flags=(), jobs=None):
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(compile_one, SOURCES))
     out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in results], "-o", LIB])
-    if verbose:
-        for _, text in results:
-            if text.strip():
-                print(text)
-        if out.strip():
-            print(out)
+    import json
+    usage = {}
+    for src, (_, text) in zip(SOURCES, results):
+        usage[src], rest = _resource_usage(text)
+        if verbose and rest.strip():
+            print(rest)
+    with open(USAGE, "w") as f:
+        json.dump(usage, f, indent=1, sort_keys=True)
+    if verbose and out.strip():
+        print(out)
     return LIB
 
 

@@ -67,8 +67,7 @@ constexpr int kMaxXcd = 16;
 
 // workspace: [0..15] ticket counters (one per XCD slot), [16] error word, [17] a tag written with every clearing
 // (ssd_params.h: kChainWsTag), [32..47] hardware id of the XCD that took each slot (+1), flags from [kWsHeaderInts]
-constexpr int kWsHeaderInts = 64, kWsErr = kChainWsErrWord, kWsTag = kChainWsTagWord, kWsOwner = 32;
-constexpr int kWsTagValue = kChainWsTag;
+constexpr int kWsHeaderInts = 64, kWsErr = kChainWsErrWord, kWsOwner = 32;
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (4 or 8); R = chunks per work item (1, 2 or 4).
 // out, initial_states and final_states are fp32.

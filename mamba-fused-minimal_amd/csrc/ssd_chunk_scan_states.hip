@@ -160,7 +160,6 @@ __global__ void __launch_bounds__(256, 2) scan_states_kernel(const ScanParams p)
     const int b = item / p.C;
     const int g = h / (p.nheads / p.ngroups);
     const int p0 = pt * 16 * PB;
-    const int tok0 = c * p.Q + wave * 16 * MB;          // first token of this wave
 
     // per-token scale of every block of this wave (kernels/ssd_chunk_scan.py:86-88, 101-104), before any request
     // that the explicit waits below count
