@@ -180,14 +180,11 @@ static hipError_t launch_t(const CumsumParams &p, hipStream_t s)
 {
     const dim3 grid((p.nheads + HT - 1) / HT, p.C, p.batch);
     const size_t lds = (size_t)HT * (p.Q + 4) * sizeof(float);
-    static bool big_lds = false;        // more than 64 KB of LDS has to be requested explicitly, once per kernel
-    if (lds > 65536 && !big_lds) {
-        hipError_t e = hipFuncSetAttribute((const void *)chunk_cumsum_kernel<EPL, VEC, HT, VLOAD>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           HT * (kMaxQ + 4) * (int)sizeof(float));
-        if (e != hipSuccess) return e;
-        big_lds = true;
-    }
+    // more than 64 KB of LDS has to be asked for, once per kernel and device
+    static std::atomic<uint64_t> configured{0};
+    const hipError_t e = ensure_dynamic_lds((const void *)chunk_cumsum_kernel<EPL, VEC, HT, VLOAD>,
+                                            lds > 65536 ? HT * (kMaxQ + 4) * (int)sizeof(float) : 0, configured);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL((chunk_cumsum_kernel<EPL, VEC, HT, VLOAD>), grid, dim3(256), lds, s, p);
     return hipGetLastError();
 }
