@@ -114,7 +114,9 @@ int ssd_state_passing_fwd(const ssd_tensor *states, const ssd_tensor *dA_chunk, 
  * that keeps every compute unit busy plus a streaming recurrence; that needs a place for the chunk states: a fp32
  * `out` serves as one (the recurrence then works in place), and so does a fp32 `states` buffer.  With a 16-bit `out`
  * and no `states` such a problem stays on the kernel with one workgroup per tile, which is slower (the library never
- * allocates): a caller in that position gains by passing `states`.
+ * allocates): a caller in that position gains by passing `states`.  Arguments that only the plain FMA kernel takes
+ * (fp32 or fp16 x / B, sizes off the MFMA tiling) run as the same two launches from two chunks upwards, given a fp32
+ * `out` or a fp32 `states`.
  */
 int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
                                       const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,

@@ -122,12 +122,23 @@ bool pair_supported(const Params &p)
 }
 
 // chunk states into p.states, then the recurrence over them into p.out / p.fin (which may be the same buffer)
-hipError_t launch_pair(const Params &p, hipStream_t s)
+hipError_t launch_pair(const Params &p, hipStream_t s, bool generic = false)
 {
     Params cs = p;
     cs.out = nullptr; cs.fin = nullptr; cs.init = nullptr;
-    const hipError_t e = ssd::launch_quad_chunk_state(cs, s);
+    const hipError_t e = generic ? ssd::launch_generic(cs, false, s) : ssd::launch_quad_chunk_state(cs, s);
     return e == hipSuccess ? ssd::launch_state_passing(pass_params_of(p), s) : e;
+}
+
+// The same for arguments only the plain FMA kernel takes (other element types, odd sizes): as a fused launch that
+// kernel has one workgroup per 16 x 64 piece of a state walk the whole sequence, as a chunk-state launch one per piece
+// and chunk -- batch 1 x 1024 tokens x 8 heads, fp32: 122 us fused, 28 + 17 us as chunk states + recurrence; 4096
+// tokens: 479 against 30 + 17.
+bool generic_pair_supported(const Params &p)
+{
+    if (!p.states || !p.out || !p.fin || p.C < 2) return false;
+    if (p.dt_states != ssd::DT_F32) return false;      // the recurrence would start from rounded states
+    return p.sst_p == p.dstate && p.so_p == p.dstate && p.sf_p == p.dstate && (!p.init || p.sin_p == p.dstate);
 }
 
 // the fused call's arguments with `out` doubling as the `states` buffer
@@ -144,7 +155,8 @@ enum Family { F_GENERIC = SSD_FAMILY_GENERIC, F_TOKEN_SPLIT = SSD_FAMILY_TOKEN_S
               F_PAIR = SSD_FAMILY_PAIR, F_CHAIN = SSD_FAMILY_CHAIN };
 struct Choice {
     int family;
-    bool states_in_out;      // F_PAIR: `out` doubles as the place for the chunk states
+    bool states_in_out;      // chunk-state launch + recurrence: `out` doubles as the place for the chunk states
+    bool generic_pair;       // F_GENERIC as chunk-state launch + recurrence
 };
 
 // The kernel family of a call without a workspace.
@@ -155,21 +167,25 @@ Choice choose(const Params &p, bool fused, int64_t n_cu)
     // kernel, which puts four waves on every tile, has the shorter chunk.
     const int tiles = p.batch * p.nheads * (p.headdim / 32);
     const int forced = g_forced_split.load(std::memory_order_relaxed);      // one value for the whole choice
-    if (fused && (forced == 1 || (forced == 0 && tiles >= 2 * n_cu)) && ssd::quad_supported(p)) return {F_FOUR_TILE, false};
+    if (fused && (forced == 1 || (forced == 0 && tiles >= 2 * n_cu)) && ssd::quad_supported(p)) return {F_FOUR_TILE, false, false};
     // Few state tiles, many chunks, fp32 `out`: the chunk-state launch keeps every compute unit busy where the
     // fused kernels have one workgroup per tile.  It writes the chunk states into `out`, and the streaming
     // recurrence turns them into the passed states in place (b=1 L=32768 H=80: 330 us against 425 us).
     if (fused && !p.states && forced == 0 && tiles < 2 * n_cu && (int64_t)tiles * p.C >= 32 * n_cu &&
         p.dt_out == ssd::DT_F32 && pair_supported(with_states_in_out(p)))
-        return {F_PAIR, true};
+        return {F_PAIR, true, false};
     // The caller wants the per-chunk states as well: the chunk-state launch of the four-tile kernel, which keeps
     // every compute unit busy whatever the number of tiles, then the streaming recurrence over what it wrote
     // (b=1 L=32768 H=80: 336 us against 496 us for the token-split kernel doing both at once).
     if (fused && p.states && (forced == 1 || (forced == 0 && (int64_t)tiles * p.C >= 32 * n_cu)) && pair_supported(p))
-        return {F_PAIR, false};
+        return {F_PAIR, false, false};
     if (!fused && (forced == 1 || (forced == 0 && (int64_t)tiles * p.C >= 8 * n_cu)) && ssd::quad_chunk_state_supported(p))
-        return {F_FOUR_TILE, false};
-    return {ssd::mfma_supported(p) ? F_TOKEN_SPLIT : F_GENERIC, false};
+        return {F_FOUR_TILE, false, false};
+    if (ssd::mfma_supported(p)) return {F_TOKEN_SPLIT, false, false};
+    if (fused && forced == 0 && !p.states && p.dt_out == ssd::DT_F32 && generic_pair_supported(with_states_in_out(p)))
+        return {F_GENERIC, true, true};
+    if (fused && forced == 0 && p.states && generic_pair_supported(p)) return {F_GENERIC, false, true};
+    return {F_GENERIC, false, false};
 }
 
 int run(const Params &p_in, bool fused, void *stream)
@@ -185,7 +201,9 @@ int run(const Params &p_in, bool fused, void *stream)
         case F_FOUR_TILE: e = fused ? ssd::launch_quad(p, s) : ssd::launch_quad_chunk_state(p, s); break;
         case F_PAIR: e = launch_pair(c.states_in_out ? with_states_in_out(p) : p, s); break;
         case F_TOKEN_SPLIT: e = ssd::launch_mfma(p, fused, s); break;
-        default: e = ssd::launch_generic(p, fused, s); break;
+        default:
+            e = c.generic_pair ? launch_pair(c.states_in_out ? with_states_in_out(p) : p, s, true) : ssd::launch_generic(p, fused, s);
+            break;
     }
     return (int)e;
 }

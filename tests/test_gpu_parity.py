@@ -86,6 +86,41 @@ def test_config0_fp32_generic_path(ops, oracle):
     _run_case(ops, oracle, oracle.make_inputs(0), name="cfg0")
 
 
+@pytest.mark.parametrize("kw", [
+    dict(),                                              # the configuration itself: fp32 inputs
+    dict(L=1000, nseq=3, init=True),                     # ragged last chunk, packed sequences, initial states
+    dict(L=300, H=3, P=40, N=24, Q=64, dtype="bf16"),    # bf16, but sizes only the plain kernel takes
+    dict(L=256),                                         # one chunk: nothing to split
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()) or "cfg0")
+def test_plain_kernel_fused_call_as_chunk_states_plus_recurrence(ops, oracle, kw):
+    # arguments only the plain FMA kernel takes: with two chunks or more the fused call runs as that kernel's chunk-state
+    # launch into `out` (or `states=`) + the recurrence in place; a forced kernel family keeps it on the fused launch.
+    # Both against the oracle (fused_globalbar.py:201-266 semantics) and against each other.
+    d = oracle.make_inputs(0, **kw)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    init, seq = _dev(d["initial_states"]), _dev(d["seq_idx"])
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"],
+                                          seq_idx=d["seq_idx"])
+    want_states = oracle.chunk_state_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], seq_idx=d["seq_idx"])
+    results = []
+    for forced in (0, 2):
+        old = ops.set_token_split(forced)
+        try:
+            out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=init, seq_idx=seq)
+            states = torch.full(want_states.shape, float("nan"), device="cuda")
+            out_s, fin_s = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=init, seq_idx=seq,
+                                                                    states=states)
+            torch.cuda.synchronize()
+        finally:
+            ops.set_token_split(old)
+        for what, got, want in (("out", out, want_out), ("final", fin, want_fin), ("out+states", out_s, want_out),
+                                ("final+states", fin_s, want_fin), ("states", states, want_states)):
+            _check(f"plain[{forced}].{what}", got, want)
+        results.append((out, fin))
+    assert float((results[0][0] - results[1][0]).abs().max()) <= 1e-4
+    assert float((results[0][1] - results[1][1]).abs().max()) <= 1e-4
+
+
 def test_config1_mamba2_130m(ops, oracle):
     _run_case(ops, oracle, oracle.make_inputs(1), name="cfg1")
 
