@@ -57,6 +57,16 @@ int check_dims(const ssd_dims *d)
 
 bool present(const ssd_tensor *t) { return t && t->data; }
 
+// A dimension of size one is only ever indexed with zero, so whatever stride the caller reports for it (frameworks
+// keep arbitrary ones on such dimensions of views) must not decide alignment checks or kernel choice: zero them.
+void drop_unit_strides(Params &p)
+{
+    if (p.batch == 1) p.sx_b = p.sB_b = p.sdt_b = p.sda_b = p.ssq_b = p.sin_b = p.sst_b = p.so_b = p.sf_b = 0;
+    if (p.nheads == 1) p.sx_h = p.sdt_h = p.sda_h = p.sin_h = p.sst_h = p.so_h = p.sf_h = 0;
+    if (p.ngroups == 1) p.sB_g = 0;
+    if (p.C == 1) p.sdt_c = p.sda_c = p.sst_c = p.so_c = 0;
+}
+
 // Fills the part of Params common to the chunk-state and fused calls.
 int fill_common(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dacs,
                 const ssd_tensor *seq, const ssd_tensor *states, const ssd_dims *d, int clamp)
@@ -87,6 +97,7 @@ int fill_common(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_t
         p.states = states->data; p.dt_states = states->dtype;
         p.sst_b = states->stride[0]; p.sst_c = states->stride[1]; p.sst_h = states->stride[2]; p.sst_p = states->stride[3];
     }
+    drop_unit_strides(p);
     return SSD_OK;
 }
 
@@ -379,6 +390,7 @@ static int fill_fused(Params &p, const ssd_tensor *x, const ssd_tensor *B, const
         p.init = initial_states->data; p.dt_init = initial_states->dtype;
         p.sin_b = initial_states->stride[0]; p.sin_h = initial_states->stride[1]; p.sin_p = initial_states->stride[2];
     }
+    drop_unit_strides(p);
     return SSD_OK;
 }
 

@@ -737,7 +737,11 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
         r = cost::chain_chunks_per_item(q, nullptr);
     }
     const int64_t total = (int64_t)n_units * ((p.C + r - 1) / r);
-    const int n_wg = (int)(total < n_cu ? total : n_cu);
+    int n_wg = (int)(total < n_cu ? total : n_cu);
+    // LOCAL: a workgroup only works on the units of the XCD it finds itself on, so every XCD needs one.  Workgroups go
+    // to the XCDs in turn, but not starting from XCD 0 (the turn carries over from the launch before): a whole number
+    // of rounds, at least one, reaches them all; workgroups without work leave at once.
+    if (local) n_wg = (n_wg + p.n_xcd - 1) / p.n_xcd * p.n_xcd;
     if (p.seq) return local ? launch_chain_t<true, true>(p, r, n_wg, s) : launch_chain_t<true, false>(p, r, n_wg, s);
     return local ? launch_chain_t<false, true>(p, r, n_wg, s) : launch_chain_t<false, false>(p, r, n_wg, s);
 }

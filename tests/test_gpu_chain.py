@@ -142,6 +142,18 @@ def test_dt_preparation_and_chain_kernel_in_one_call(ops, oracle, kw, kernel):
         assert torch.equal(dt2, dt) and torch.equal(dA2, dA) and torch.equal(out2, out) and torch.equal(fin2, fin)
 
 
+def test_chain_local_with_fewer_units_than_xcds(ops, oracle):
+    # One unit (two heads), per-XCD tickets insisted on: the unit belongs to one XCD, and that XCD must get a workgroup
+    # whichever XCD the launch happens to start its round of workgroups on -- small launches in front move that turn.
+    # (A launch of as many workgroups as work items, two here, once left the unit's XCD without one: every output
+    # wrong and no error reported.)
+    d = oracle.make_inputs(2, b=1, L=1730, H=2, init=True)
+    for i in range(12):
+        for _ in range(i):
+            torch.zeros(64 * (i + 1), device="cuda")          # a one-workgroup launch each
+        _chain_case(ops, oracle, d, LOCAL, 4, f"chain.local.one_unit[{i}]")
+
+
 def test_chain_matches_the_other_fused_kernels(ops, oracle):
     # same inputs through the chain kernel and through the kernel the workspace-less entry point picks
     d = oracle.make_inputs(2, b=2, L=4096, H=16)
