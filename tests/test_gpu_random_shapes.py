@@ -60,3 +60,54 @@ def test_random_shape(ops, oracle, seed):
             err = (got - want).abs()
             bad = int((err > ATOL + RTOL * want.abs()).sum())
             assert bad == 0, f"seed {seed} {kw} {name}.{what}: {bad} mismatches, max abs err {float(err.max()):.3e}"
+
+
+def _draw_any(seed):
+    """Anything the entry points accept: element types, sizes off every tiling, strided chunk-end decay."""
+    rng = random.Random(7000 + seed)
+    G = rng.choice([1, 1, 2, 3])
+    kw = dict(b=rng.choice([1, 2, 3]), H=G * rng.choice([1, 2, 4, 5]), G=G, P=rng.choice([16, 32, 40, 64, 128]),
+              N=rng.choice([16, 24, 64, 128]), Q=rng.choice([64, 128, 256]), init=rng.random() < 0.5,
+              dtype=rng.choice(["bf16", "bf16", "fp32", "fp16"]))
+    kw["L"] = rng.randrange(kw["Q"] // 2, 6 * kw["Q"])         # 1 .. 6 chunks, the single one possibly short
+    if rng.random() < 0.4 and kw["L"] > 600:
+        kw["nseq"] = rng.randrange(2, 5)
+    return kw, rng.choice([torch.float32, torch.float32, torch.bfloat16]), rng.random() < 0.5
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_arguments_without_a_workspace(ops, oracle, seed):
+    # the three entry points of the path on whatever the draw gives: fused (with and without a `states` output, fp32 or
+    # bf16 passed states), chunk state, state passing -- every kernel family is somebody's fallback here
+    kw, out_dtype, with_states = _draw_any(seed)
+    d = oracle.make_inputs(3 if "nseq" in kw else 1, **kw)
+    x, B, dt, dA, seq, init = d["x"], d["B"], d["dt"], d["dA_cumsum"], d["seq_idx"], d["initial_states"]
+    print(f"[random-any {seed}] {kw} out {out_dtype} states {with_states}", flush=True)
+    want_states = oracle.chunk_state_ref(B, x, dt, dA, seq_idx=seq)
+    want_out, want_fin = oracle.fused_ref(B, x, dt, dA, initial_states=init, seq_idx=seq)
+    xd, Bd, dtd, dAd, seqd, initd = map(_dev, (x, B, dt, dA, seq, init))
+    b, L, H, P = x.shape
+    N, C = B.shape[-1], dt.shape[2]
+
+    def check(what, got, want, rtol=RTOL, atol=ATOL):
+        got = got.float().cpu()
+        assert got.shape == want.shape and torch.isfinite(got).all(), (seed, what)
+        err = (got - want.float()).abs()
+        bad = int((err > atol + rtol * want.abs()).sum())
+        assert bad == 0, f"seed {seed} {kw} {what}: {bad} mismatches, max abs err {float(err.max()):.3e}"
+
+    st_buf = torch.full((b, C, H, P, N), float("nan"), device="cuda") if with_states else None
+    out, fin = ops._fused_chunk_state_state_passing_fwd(Bd, xd, dtd, dAd, out_dtype, initial_states=initd, seq_idx=seqd,
+                                                        states=st_buf)
+    torch.cuda.synchronize()
+    check("out", out, want_out, *((1e-2, 1e-3) if out_dtype != torch.float32 else (RTOL, ATOL)))
+    check("final", fin, want_fin)
+    if with_states:
+        check("states", st_buf, want_states)
+    st = ops._chunk_state_fwd(Bd, xd, dtd, dAd, seq_idx=seqd)
+    check("chunk_state", st, want_states)
+    o2, f2 = ops._state_passing_fwd(st.flatten(-2), dAd[:, :, :, -1], initial_states=None if initd is None else initd.flatten(-2),
+                                    seq_idx=seqd, chunk_size=dt.shape[-1])
+    torch.cuda.synchronize()
+    check("state_passing.out", o2.reshape(b, C, H, P, N), want_out)
+    check("state_passing.final", f2.reshape(b, H, P, N), want_fin)
