@@ -111,3 +111,41 @@ def test_random_arguments_without_a_workspace(ops, oracle, seed):
     torch.cuda.synchronize()
     check("state_passing.out", o2.reshape(b, C, H, P, N), want_out)
     check("state_passing.final", f2.reshape(b, H, P, N), want_fin)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_neighbours_of_the_path(ops, oracle, seed):
+    # the producer of dt / dA_cumsum (kernels/ssd_chunk_state.py:33-79) and the consumer of the passed states
+    # (kernels/ssd_chunk_scan.py:94-117) on drawn sizes and element types, both matrix-core scan kernels in turn
+    kw, _, _ = _draw_any(seed + 100)
+    d = oracle.make_inputs(3 if "nseq" in kw else 1, **kw)
+    Q = d["cfg"]["Q"]
+    rng = random.Random(seed)
+    softplus, use_bias = rng.random() < 0.6, rng.random() < 0.6
+    limit = rng.choice([(0.0, float("inf")), (2e-3, 5e-2)])
+    raw, A, bias = d["dt_raw"], d["A"], d["dt_bias"] if use_bias else None
+    print(f"[random-neighbours {seed}] {kw} softplus {softplus} bias {use_bias} limit {limit}", flush=True)
+    want_da, want_dt = oracle.chunk_cumsum_ref(raw, A, Q, dt_bias=bias, dt_softplus=softplus, dt_limit=limit)
+    got_da, got_dt = ops._chunk_cumsum_fwd(_dev(raw), _dev(A), Q, dt_bias=_dev(bias), dt_softplus=softplus, dt_limit=limit)
+    torch.cuda.synchronize()
+
+    def check(what, got, want, rtol, atol):
+        got = got.float().cpu()
+        assert got.shape == want.shape and torch.isfinite(got).all(), (seed, what)
+        err = (got - want.float()).abs()
+        bad = int((err > atol + rtol * want.abs()).sum())
+        assert bad == 0, f"seed {seed} {kw} {what}: {bad} mismatches, max abs err {float(err.max()):.3e}"
+
+    check("cumsum.dt", got_dt, want_dt, 2e-6, 1e-9)
+    check("cumsum.dA_cumsum", got_da, want_da, 1e-5, 1e-6)
+    seq, dA = d["seq_idx"], d["dA_cumsum"]
+    prev, _ = oracle.fused_ref(d["B"], d["x"], d["dt"], dA, initial_states=d["initial_states"], seq_idx=seq)
+    want_y = oracle.chunk_scan_states_ref(d["C"], prev, dA, seq_idx=seq)
+    for kernel in (1, 2):
+        old = ops.set_scan_kernel(kernel)
+        try:
+            y = ops._chunk_scan_states_fwd(_dev(d["C"]), _dev(prev), _dev(dA), seq_idx=_dev(seq), out_dtype=torch.float32)
+            torch.cuda.synchronize()
+        finally:
+            ops.set_scan_kernel(old)
+        check(f"scan_states[{kernel}]", y, want_y, RTOL, ATOL)
