@@ -234,3 +234,29 @@ def test_chain_back_to_back_and_other_stream(ops, oracle):
         assert torch.equal(out, results[0][0]) and torch.equal(fin, results[0][1])
     want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
     assert _mismatches(results[0][0], want_out)[0] == 0 and _mismatches(results[0][1], want_fin)[0] == 0
+
+
+@pytest.mark.parametrize("kernel", [LOCAL, GLOBAL], ids=["local", "global"])
+def test_chain_launches_competing_for_the_compute_units(ops, oracle, kernel):
+    # Two streams, each with chain launches that want every compute unit for themselves (one workgroup fills a compute
+    # unit: registers and LDS), a workspace each: workgroups of one launch start as those of the other leave, so neither
+    # launch has all its workgroups resident -- the case the ticket order is for (an item only waits for smaller
+    # tickets, and tickets are drawn by running workgroups).  Every result must be right and no wait may run out.
+    d = oracle.make_inputs(2, b=2, L=8192, H=40)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    initd = _dev(d["initial_states"])
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    spaces = [torch.empty(1 << 18, dtype=torch.int32, device="cuda") for _ in streams]
+    results = [[], []]
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                results[i].append(ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=initd,
+                                                                           _kernel=kernel, _workspace=spaces[i]))
+    torch.cuda.synchronize()
+    for i, st in enumerate(streams):
+        assert ops._fused_workspace_status(spaces[i]) == 0
+        for out, fin in results[i]:
+            assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
