@@ -139,7 +139,7 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  *
  * workspace: device memory, 4-byte aligned, at least ssd_fused_workspace_bytes(dims); the call clears what it uses
  * (a small fill launch, no memset node), so the memory may hold anything and may be reused by later calls on the
- * same stream.  Two calls whose kernels may overlap (different streams) need workspaces of their own.
+ * same stream (a caller that keeps a workspace to itself can save the fill launch: `epoch` below).  Two calls whose kernels may overlap (different streams) need workspaces of their own.
  * kernel: SSD_KERNEL_AUTO lets the library choose between this kernel and those of ssd_fused_chunk_state_passing_fwd
  * (which it runs when the shape, element types or a `states` output rule the chain kernel out: it needs bf16 x / B,
  * fp32 out / initial / final states, no `states`, dstate 64 or 128, chunk 128 or 256); SSD_KERNEL_CHAIN insists on it
@@ -155,7 +155,15 @@ typedef struct ssd_fused_opts {
     int32_t spin_limit;       /* flag polls before a wave gives up; 0 = default (about 4 million) */
     int32_t kernel;           /* SSD_KERNEL_AUTO, or one of the SSD_KERNEL_CHAIN values to insist on that kernel */
     int32_t chunks_per_item;  /* chain kernel: consecutive chunks per work item, 1, 2 or 4; 0 = choose */
-    int32_t reserved;
+    int32_t epoch;            /* chain kernel: 0 = the workspace may hold anything, the call clears it with a small fill
+                                 launch (default).  n > 0 = a promise that saves that launch: the call before this one on
+                                 this workspace (same stream, or ordered before it) was made with epoch n - 1, or with
+                                 epoch 0 if n == 2, and no other use of the memory came in between.  Flags carry the
+                                 epoch and the ticket counters exist once per parity, so the kernel leaves what the next
+                                 epoch needs at zero by itself.  Only calls that ran the chain kernel count (see
+                                 used_workspace).  Start again from 0 before n would overflow. */
+    int32_t *used_workspace;  /* host memory or NULL: set to 1 if the call ran the chain kernel -- and so used the
+                                 workspace and its epoch --, to 0 if another kernel family served it */
 } ssd_fused_opts;
 
 enum { SSD_KERNEL_AUTO = 0, SSD_KERNEL_CHAIN = 1, SSD_KERNEL_CHAIN_LOCAL = 2, SSD_KERNEL_CHAIN_GLOBAL = 3 };
@@ -185,7 +193,7 @@ int ssd_fused_workspace_status(const void *workspace, void *stream);
  * ends); the call clears what it uses with a small fill launch and runs the chain kernel, whatever the problem size
  * (the kernel choice of the other entry points is not made here: SSD_ERR_SHAPE for arguments that kernel does not
  * cover -- it needs bf16 x / B, fp32 out / initial / final states, dstate 64 or 128, chunk 128 or 256 --,
- * SSD_ERR_SCRATCH when batch * nheads * (headdim / 32) * nchunks + 64 flags do not fit the array, i.e. above 262 080
+ * SSD_ERR_SCRATCH when batch * nheads * (headdim / 32) * nchunks + 128 ints do not fit the array, i.e. above 262 016
  * (state tile, chunk) pairs).  Every call on a GPU shares that GPU's array: two calls whose kernels may overlap
  * (different streams, different host threads) race on it and must be serialised by the caller.
  * ssd_fused_static_status is ssd_fused_workspace_status for that array.

@@ -287,6 +287,7 @@ bool chain_preferred(const Params &p, int n_cu)
 int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *opts, bool *use)
 {
     *use = false;
+    if (opts && opts->used_workspace) *opts->used_workspace = 0;
     const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
     if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
     const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
@@ -294,6 +295,7 @@ int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *
     if (have_ws && ssd::chain_supported(p) &&
         (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
         *use = true;
+        if (opts->used_workspace) *opts->used_workspace = 1;
         return check_device();
     }
     return kernel != SSD_KERNEL_AUTO ? SSD_ERR_SCRATCH : SSD_OK;     // forced, but no workspace or not a shape it covers
@@ -302,6 +304,7 @@ int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *
 int run_chain(Params &p, const ssd_fused_opts *opts, void *stream)
 {
     p.ws = (int *)opts->workspace;
+    p.epoch = opts->epoch > 0 ? opts->epoch : 0;
     p.spin_limit = opts->spin_limit;
     p.n_seg = opts->chunks_per_item == 1 || opts->chunks_per_item == 2 || opts->chunks_per_item == 4 ? opts->chunks_per_item : 0;
     return (int)ssd::launch_chain(p, compute_units(),
@@ -462,14 +465,14 @@ int ssd_fused_workspace_status(const void *workspace, void *stream)
     if (!workspace) return SSD_ERR_NULL;
     int rc = check_device();
     if (rc) return rc;
-    static_assert(ssd::kChainWsTagWord == ssd::kChainWsErrWord + 1, "read in one copy");
-    int word[2] = {0, 0};       // error word and tag, behind the sixteen ticket counters
+    static_assert(ssd::kChainWsEpochWord == ssd::kChainWsErrWord + 2 && ssd::kChainWsTagWord == ssd::kChainWsErrWord + 3, "read in one copy");
+    int word[4] = {0, 0, 0, 0};       // error words of both parities, epoch of the last launch, tag
     hipError_t e = hipMemcpyAsync(word, (const int *)workspace + ssd::kChainWsErrWord, sizeof(word), hipMemcpyDeviceToHost,
                                   (hipStream_t)stream);
     if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return (int)e;
-    if (word[1] != ssd::kChainWsTag) return SSD_OK;      // the chain kernel has not run on this memory: nothing to report
-    return word[0] ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
+    if (word[3] != ssd::kChainWsTag) return SSD_OK;      // the chain kernel has not run on this memory: nothing to report
+    return word[word[2] & 1] ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
 }
 
 int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
@@ -509,7 +512,7 @@ int ssd_fused_cumsum_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_t
     // the four-tile kernel, 232 against 197 in the chain kernel): their workgroups take two heads each and have to
     // gather those two columns out of the token-major dt rows, a cache line per token, where the producer reads the
     // rows whole.
-    if (chain) {
+    if (chain && opts->epoch <= 0) {
         cp.clear = (int *)opts->workspace;
         cp.n_clear = (int)(ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks) / sizeof(int));
         p.ws_cleared = 1;

@@ -65,9 +65,8 @@ template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * N
 constexpr int kAuxDevice = 16;      // sc1
 constexpr int kMaxXcd = 16;
 
-// workspace: [0..15] ticket counters (one per XCD slot), [16] error word, [17] a tag written with every clearing
-// (ssd_params.h: kChainWsTag), [32..47] hardware id of the XCD that took each slot (+1), flags from [kWsHeaderInts]
-constexpr int kWsHeaderInts = 64, kWsErr = kChainWsErrWord, kWsOwner = 32;
+// workspace layout: ssd_params.h
+constexpr int kWsHeaderInts = kChainWsHeaderInts, kWsOwner = kChainWsOwnerWord;
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (4 or 8); R = chunks per work item (1, 2 or 4).
 // out, initial_states and final_states are fp32.
@@ -114,7 +113,9 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     const int n_pt = p.headdim >> 5;
     const int L = p.seqlen, C = p.C;
     const int64_t xrb = 2 * p.sx_l, Brb = 2 * p.sB_l;            // row pitch in bytes
-    int *const ws_ticket = p.ws + slot, *const ws_err = p.ws + kWsErr, *const ws_flags = p.ws + kWsHeaderInts;
+    const int epoch = p.epoch, bank = epoch & 1;
+    int *const ws_ticket = p.ws + kChainWsBankStride * bank + slot, *const ws_err = p.ws + kChainWsErrWord + bank;
+    int *const ws_flags = p.ws + kWsHeaderInts;
 
     // ---- work items ------------------------------------------------------------------------------------------
     // A workgroup walks a stream of chunks: the R chunks of its current item, then those of the next.  `Item` is one
@@ -336,8 +337,8 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     auto load_flag = [&](const int *f) { return __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     auto raise_flag = [&](int *f) {
         if (lane == 0) {
-            if (LOCAL) *(volatile int *)f = 1;
-            else __hip_atomic_store(f, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (LOCAL) *(volatile int *)f = epoch;
+            else __hip_atomic_store(f, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
     // I: the last chunk of the item (chunks I.c - I.r .. I.c)
@@ -414,7 +415,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         if (use_prev && c0 > 0) {
             // out[:, c0] of this tile is complete once its flag is up
             int polls = 0;
-            while (load_flag(flag + c0) == 0) {
+            while (load_flag(flag + c0) != epoch) {
                 __builtin_amdgcn_s_sleep(1);
                 if (++polls >= p.spin_limit) {
                     if (lane == 0) __hip_atomic_fetch_or(ws_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -474,6 +475,14 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         const bool single = !(R > 1 && c_first + 1 < C);
         tq[0] = t;
         tq[1] = single ? __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -1;
+        if (t == 0 && slot == 0) {
+            // one thread per launch: what the next launch on this workspace (epoch + 1, the other parity) must find
+            // at zero -- nothing of it is touched by this launch
+            int *const other = p.ws + kChainWsBankStride * (bank ^ 1);
+            for (int i = 0; i < kMaxXcd; ++i) __hip_atomic_store(other + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(p.ws + kChainWsErrWord + (bank ^ 1), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(p.ws + kChainWsEpochWord, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     // rows past the end of the sequence are not fetched and leave their LDS slots untouched; their weight is zero,
     // so the slots only have to hold finite numbers
@@ -710,7 +719,10 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     if (p.spin_limit <= 0) p.spin_limit = 1 << 22;
     const int64_t n_ws = chain::kWsHeaderInts + (int64_t)p.n_items * p.C;
     hipError_t e = hipSuccess;
-    if (!p.ws_cleared) {
+    // epoch <= 0: the workspace may hold anything: cleared here (or by the launch in front), and this is launch 1 on it
+    const bool clear = p.epoch <= 0;
+    if (clear) p.epoch = 1;
+    if (clear && !p.ws_cleared) {
         hipLaunchKernelGGL(chain::clear_kernel, dim3((unsigned)((n_ws + 255) / 256 < 1024 ? (n_ws + 255) / 256 : 1024)), dim3(256), 0, s,
                            p.ws, (int)n_ws);
         e = hipGetLastError();

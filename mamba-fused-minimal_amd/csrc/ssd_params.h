@@ -40,6 +40,7 @@ struct Params {
     int n_xcd;            // XCDs (L2 caches) the units of that kernel are dealt to
     int n_cu;             // compute units of the device (0: not known, the launchers then assume 256 in 8 XCDs)
     int ws_cleared;       // the launch in front of that kernel has cleared `ws` already (chain_workspace_clear below)
+    int epoch;            // of this launch on `ws` (below); <= 0: contents unknown, the launcher clears it and takes 1
 };
 
 // State passing on a flattened state axis.
@@ -168,9 +169,18 @@ hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
 bool chain_supported(const Params &p);
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
 
-// Words of a chain workspace that the host reads back: the error word, and behind it a tag that every launch of the
-// chain kernel writes when it clears the workspace -- without it the error word is whatever the memory held.
-constexpr int kChainWsErrWord = 16, kChainWsTagWord = 17, kChainWsTag = 0x53534443;
+// Layout of a chain workspace (ints).  A launch carries an epoch, one more than that of the launch before it on the
+// same workspace.  Everything a launch must find in a known state is either tagged with the epoch or kept twice:
+//   [32 b + slot]  ticket counters, one bank b = epoch & 1 per parity, a slot per XCD (16).  The workgroup that draws
+//                  ticket 0 of slot 0 zeroes the other bank, the other error word and records the epoch: the next
+//                  launch finds its counters at zero without a fill launch in between.
+//   [64 + b]       error word of the launch with parity b;  [66] epoch of the last launch;  [67] a tag that says a
+//                  chain launch has cleared this memory at least once (without it the words above mean nothing)
+//   [96 + slot]    hardware id (+1) of the XCD that drew from each slot
+//   [128 ...]      flags, one per (state tile, chunk): raised = holds the epoch of the launch (older values, from
+//                  launches before, and the zeros of a clearing never equal it)
+constexpr int kChainWsHeaderInts = 128, kChainWsBankStride = 32, kChainWsErrWord = 64, kChainWsEpochWord = 66,
+              kChainWsTagWord = 67, kChainWsOwnerWord = 96, kChainWsTag = 0x53534443;
 // The value a cleared chain workspace holds at int i: zero, except for the tag.  Any kernel that runs in front of the
 // chain kernel on the same stream may do the clearing (the stand-alone producer of dt / dA_cumsum does when both are
 // launched by one call); Params::ws_cleared then keeps the chain kernel's own fill launch away.

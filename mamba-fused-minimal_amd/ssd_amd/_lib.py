@@ -30,7 +30,7 @@ class SsdDims(ctypes.Structure):
 
 class SsdFusedOpts(ctypes.Structure):
     _fields_ = [("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64), ("spin_limit", ctypes.c_int32),
-                ("kernel", ctypes.c_int32), ("chunks_per_item", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("kernel", ctypes.c_int32), ("chunks_per_item", ctypes.c_int32), ("epoch", ctypes.c_int32), ("used_workspace", ctypes.POINTER(ctypes.c_int32))]
 
 
 class SsdFusedPlan(ctypes.Structure):

@@ -9,6 +9,7 @@ of the reference.  The wrappers own allocation and argument checking; the arithm
 kernels behind the C ABI of libssd_gfx950.so, asynchronously on the current torch stream."""
 import ctypes
 import math
+import threading
 
 import torch
 
@@ -17,6 +18,31 @@ from . import _lib
 
 def _stream(t):
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+# Workspaces of the ticket / flag-chain kernel that the wrappers keep to themselves: one per (device, stream), grown on
+# demand, with the epoch of the last launch on it.  A workspace nobody else writes to lets a call tell the library that
+# the launch before left it in order (ssd_fused_opts.epoch), which saves the fill launch in front of the kernel.
+_WORKSPACES = {}
+_WORKSPACES_LOCK = threading.Lock()
+
+
+def _own_workspace(x, nbytes):
+    """-> (int32 tensor, epoch to pass).  Call with _WORKSPACES_LOCK held, and keep it until the launch is enqueued:
+    the epochs must reach the stream in order."""
+    stream = torch.cuda.current_stream(x.device)
+    if torch.cuda.is_current_stream_capturing():
+        # a captured launch is replayed with the same arguments: the same epoch again and again would take the flags of
+        # the replay before for its own.  Epoch 0 (clear every time) is what a graph needs.
+        return torch.empty(((nbytes + 3) // 4,), device=x.device, dtype=torch.int32), 0
+    key = (x.device.index, stream.cuda_stream)
+    ent = _WORKSPACES.get(key)
+    if ent is None or ent[0].numel() * 4 < nbytes:
+        ent = [torch.empty((max(nbytes, 1 << 16) + 3) // 4, device=x.device, dtype=torch.int32), 0]
+        _WORKSPACES[key] = ent
+    ent[1] = 0 if ent[1] >= (1 << 30) else ent[1]
+    epoch = 0 if ent[1] == 0 else ent[1] + 1
+    return ent, epoch
 
 
 def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
@@ -104,7 +130,7 @@ def _state_passing_fwd(states, dA_chunk_cumsum, initial_states=None, seq_idx=Non
 
 def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial_states=None, seq_idx=None,
                                          states=None, states_in_fp32=True, _clamp=True, _kernel=0, _spin_limit=0,
-                                         _workspace=None, _chunks_per_item=0):
+                                         _workspace=None, _chunks_per_item=0, _epoch=0):
     """One launch for chunk state + state passing.  Returns (out (b,C,H,P,N) out_dtype, final_states (b,H,P,N) fp32).
 
     Unlike the reference's fused wrappers, the per-chunk states are an internal quantity that never reaches
@@ -115,7 +141,9 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     flags of the kernel that spreads a sequence's chunks over all compute units.  ``_kernel`` (0 = let the library
     choose, 1 = insist on that kernel, 2 / 3 = and on its per-XCD / device-wide variant), ``_chunks_per_item``
     (1, 2 or 4 consecutive chunks per work item of that kernel, 0 = choose), ``_spin_limit`` (polls before a flag wait gives up, 0 = default) and
-    ``_workspace`` (an int32 tensor to use instead of allocating one) are test and tuning hooks."""
+    ``_workspace`` (an int32 tensor to use instead of the wrapper's own, which it keeps per device and stream and whose
+    fill launch it saves from the second call on) with ``_epoch`` (ssd_fused_opts.epoch for that tensor) are test and
+    tuning hooks."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = B.shape
@@ -143,16 +171,32 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     if initial_states is not None and initial_states.stride(-1) != 1:
         initial_states = initial_states.contiguous()
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
-    if _workspace is None:
-        _workspace = torch.empty(((int(lib.ssd_fused_workspace_bytes(dims)) + 3) // 4,), device=x.device, dtype=torch.int32)
-    opts = _lib.SsdFusedOpts(_workspace.data_ptr(), _workspace.numel() * 4, int(_spin_limit), int(_kernel),
-                             int(_chunks_per_item), 0)
-    with torch.cuda.device(x.device):
-        rc = lib.ssd_fused_chunk_state_passing_fwd_ws(
-            _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),
-            _lib.tensor_arg(seq_idx), _lib.tensor_arg(initial_states), _lib.tensor_arg(states),
-            _lib.tensor_arg(out), _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, ctypes.byref(opts),
-            _stream(x))
+
+    used = ctypes.c_int32(0)
+
+    def launch(workspace, epoch):
+        opts = _lib.SsdFusedOpts(workspace.data_ptr(), workspace.numel() * 4, int(_spin_limit), int(_kernel),
+                                 int(_chunks_per_item), int(epoch), ctypes.pointer(used))
+        with torch.cuda.device(x.device):
+            return lib.ssd_fused_chunk_state_passing_fwd_ws(
+                _lib.tensor_arg(x), _lib.tensor_arg(B), _lib.tensor_arg(dt), _lib.tensor_arg(dA_cumsum),
+                _lib.tensor_arg(seq_idx), _lib.tensor_arg(initial_states), _lib.tensor_arg(states),
+                _lib.tensor_arg(out), _lib.tensor_arg(final_states), dims, 1 if _clamp else 0, ctypes.byref(opts),
+                _stream(x))
+
+    if _workspace is not None:
+        rc = launch(_workspace, _epoch)
+    else:
+        with _WORKSPACES_LOCK:
+            ent, epoch = _own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)))
+            if isinstance(ent, list):
+                rc = launch(ent[0], epoch)
+                if rc:
+                    ent[1] = 0                            # after a failed call the contents count as unknown
+                elif used.value:
+                    ent[1] = max(epoch, 1)                # only a call that ran the chain kernel used the epoch
+            else:
+                rc = launch(ent, 0)
     _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states
 
@@ -291,14 +335,31 @@ def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dty
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
     T = _lib.tensor_arg
     lib = _lib.load()
-    if _workspace is None:
-        _workspace = torch.empty(((int(lib.ssd_fused_workspace_bytes(dims)) + 3) // 4,), device=x.device, dtype=torch.int32)
-    opts = _lib.SsdFusedOpts(_workspace.data_ptr(), _workspace.numel() * 4, 0, int(_kernel), int(_chunks_per_item), 0)
-    with torch.cuda.device(x.device):
-        rc = lib.ssd_fused_cumsum_chunk_state_passing_fwd_ws(
-            T(x), T(B), T(dt), T(A), T(dt_bias), T(seq_idx), T(initial_states), T(dt_out), T(dA_cumsum), T(out),
-            T(final_states), dims, int(bool(dt_softplus)), float(dt_limit[0]), float(dt_limit[1]), 1 if _clamp else 0,
-            ctypes.byref(opts), _stream(x))
+
+    used = ctypes.c_int32(0)
+
+    def launch(workspace, epoch):
+        opts = _lib.SsdFusedOpts(workspace.data_ptr(), workspace.numel() * 4, 0, int(_kernel), int(_chunks_per_item), int(epoch),
+                                 ctypes.pointer(used))
+        with torch.cuda.device(x.device):
+            return lib.ssd_fused_cumsum_chunk_state_passing_fwd_ws(
+                T(x), T(B), T(dt), T(A), T(dt_bias), T(seq_idx), T(initial_states), T(dt_out), T(dA_cumsum), T(out),
+                T(final_states), dims, int(bool(dt_softplus)), float(dt_limit[0]), float(dt_limit[1]), 1 if _clamp else 0,
+                ctypes.byref(opts), _stream(x))
+
+    if _workspace is not None:
+        rc = launch(_workspace, 0)
+    else:
+        with _WORKSPACES_LOCK:
+            ent, epoch = _own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)))
+            if isinstance(ent, list):
+                rc = launch(ent[0], epoch)
+                if rc:
+                    ent[1] = 0
+                elif used.value:
+                    ent[1] = max(epoch, 1)
+            else:
+                rc = launch(ent, 0)
     _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd_ws")
     return out, final_states, dA_cumsum, dt_out
 

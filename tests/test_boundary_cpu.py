@@ -100,7 +100,7 @@ def test_argument_validation_from_two_threads_with_different_hooks(lib):
     bad = _lib.dims_arg(1, 256, 3, 64, 128, 2, 256, 1)
     big = _lib.dims_arg(4, 8192, 80, 64, 128, 1, 256, 32)
     want_ws = lib.ssd_fused_workspace_bytes(big)
-    assert want_ws == 4 * (64 + 4 * 80 * 2 * 32)
+    assert want_ws == 4 * (128 + 4 * 80 * 2 * 32)
     settings = {"a": (2, 3, 1), "b": (4, 5, 2)}
     seen = {"split": {0, 2, 4}, "segment": {0, 3, 5}, "scan": {0, 1, 2}}
     errors = []

@@ -10,21 +10,53 @@ reports and still raises its flag, and the cut of an item at a sequence start.  
 time by an adversarial (seeded random) scheduler with a limit on how many may be resident, down to one -- the hardware
 promises nothing about residency.  Checked: every launch drains, every passed state equals the serial recurrence
 (ssd_state_passing.py:69-84 on scalars), no wait gives up when the limit is generous, and a limit of one poll is
-reported while the launch still drains."""
+reported while the launch still drains.  A workspace may be kept from launch to launch without clearing: flags hold the
+epoch they were raised in, ticket counters and error words exist once per parity of the epoch, and the workgroup that
+draws ticket 0 zeroes the other parity's for the launch after it (the last test)."""
 import random
 
 import pytest
 
 
+class Workspace:
+    """What survives from launch to launch when the caller keeps a workspace and passes epochs (ssd_fused_opts.epoch):
+    two banks of ticket counters and two error words, by parity of the epoch; the epoch of the last launch; flags that
+    hold the epoch they were raised in.  Cleared = all zero."""
+
+    def __init__(self, n_flags=4096):
+        self.tickets = [0, 0]
+        self.errors = [0, 0]
+        self.last_epoch = 0
+        self.flags = [0] * n_flags
+
+    def status(self):
+        return self.errors[self.last_epoch & 1]
+
+
+class _Flags:
+    """One unit's row of flags inside the workspace: truthy = raised in the current epoch."""
+
+    def __init__(self, ws, base, epoch):
+        self.ws, self.base, self.epoch = ws, base, epoch
+
+    def __getitem__(self, c):
+        return self.ws.flags[self.base + c] == self.epoch
+
+    def __setitem__(self, c, v):
+        assert v == 1
+        self.ws.flags[self.base + c] = self.epoch
+
+
 class Launch:
-    def __init__(self, n_units, C, R, n_wg, resident, spin_limit, seed, boundaries=()):
+    def __init__(self, n_units, C, R, n_wg, resident, spin_limit, seed, boundaries=(), ws=None, epoch=1):
         self.n_units, self.C, self.R, self.n_wg, self.resident, self.spin_limit = n_units, C, R, n_wg, resident, spin_limit
         self.rng = random.Random(seed)
         self.n_super = (C + R - 1) // R
         self.total = n_units * self.n_super
-        self.ticket = 0
-        self.error = 0
-        self.flag = [[0] * (C + 1) for _ in range(n_units)]
+        self.ws = ws if ws is not None else Workspace()
+        self.epoch, self.bank = epoch, epoch & 1
+        assert n_units * (C + 1) <= len(self.ws.flags)
+        self.flag = [_Flags(self.ws, u * (C + 1), epoch) for u in range(n_units)]
         # per (unit, chunk): chunk state S and decay d (zero where a sequence starts)
         self.S = [[self.rng.uniform(-1, 1) for _ in range(C)] for _ in range(n_units)]
         self.d = [[0.0 if (u, c) in boundaries else self.rng.uniform(0.1, 0.9) for c in range(C)] for u in range(n_units)]
@@ -32,9 +64,26 @@ class Launch:
         self.out = [[None] * (C + 1) for _ in range(n_units)]       # out[u][c] = state entering chunk c; [C] = final
         self.events = 0
 
+    @property
+    def ticket(self):
+        return self.ws.tickets[self.bank]
+
+    @property
+    def error(self):
+        return self.ws.errors[self.bank]
+
+    @error.setter
+    def error(self, v):
+        self.ws.errors[self.bank] = v
+
     def draw(self):
-        t = self.ticket
-        self.ticket += 1
+        t = self.ws.tickets[self.bank]
+        self.ws.tickets[self.bank] += 1
+        if t == 0:
+            # one workgroup per launch: what the next epoch (the other parity) must find at zero
+            self.ws.tickets[self.bank ^ 1] = 0
+            self.ws.errors[self.bank ^ 1] = 0
+            self.ws.last_epoch = self.epoch
         return t
 
     def item(self, t):
@@ -165,7 +214,31 @@ def test_a_wait_that_runs_out_is_reported_and_the_launch_still_drains(resident):
         L = Launch(3, 16, 1, 16, resident, spin_limit=1, seed=seed).run()
         reported += L.error
         for u in range(3):
-            assert L.flag[u][16] == 0 and all(L.flag[u][c] for c in range(1, 16))     # every flag was raised all the same
+            assert not L.flag[u][16] and all(L.flag[u][c] for c in range(1, 16))     # every flag was raised all the same
     assert reported > 0
     # and with one resident workgroup nothing ever waits: it meets its own finished items
     assert Launch(3, 16, 1, 16, 1, spin_limit=1, seed=0).run().error == 0
+
+
+def test_a_workspace_kept_from_launch_to_launch_with_epochs():
+    # no clearing between launches: shapes, chunks per item and residency change, one launch has a wait that runs out;
+    # every launch drains, computes the serial recurrence, and reports its own error word only
+    rng = random.Random(5)
+    ws = Workspace()
+    epoch = 1
+    for i in range(40):
+        n_units, C, R, n_wg = rng.choice(SHAPES)
+        limit = 1 if i % 9 == 4 else 1 << 30
+        resident = rng.choice([1, 2, 3, 1000])
+        boundaries = {(rng.randrange(n_units), rng.randrange(C)) for _ in range((n_units * C) // 7)} if i % 2 else set()
+        L = Launch(n_units, C, R, n_wg, resident, spin_limit=limit, seed=100 + i, boundaries=boundaries, ws=ws, epoch=epoch).run()
+        assert ws.last_epoch == epoch
+        assert L.ticket >= L.total
+        if limit > 1:
+            assert ws.status() == 0, i
+            want = L.reference()
+            for u in range(n_units):
+                for c in range(C + 1):
+                    assert abs(L.out[u][c] - want[u][c]) <= 1e-12 * max(1.0, abs(want[u][c])), (i, u, c)
+        epoch += 1
+    assert ws.tickets[epoch & 1] == 0            # the bank of the launch that would come next is clean

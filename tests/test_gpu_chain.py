@@ -260,3 +260,65 @@ def test_chain_launches_competing_for_the_compute_units(ops, oracle, kernel):
         assert ops._fused_workspace_status(spaces[i]) == 0
         for out, fin in results[i]:
             assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+def test_chain_workspace_kept_across_calls_with_epochs(ops, oracle):
+    # ssd_fused_opts.epoch: a workspace that only these calls touch, cleared once (epoch 0) and from then on told its
+    # epoch (2, 3, ...): no fill launch, flags carry the epoch, ticket counters alternate between two banks.  Shapes,
+    # chunks per item and the way states cross compute units change from call to call; every call against the oracle.
+    cases = [(dict(b=2, L=2048, H=8, init=True), LOCAL, 4), (dict(L=2000, H=8, nseq=5, init=True), GLOBAL, 2),
+             (dict(L=2304, H=8), LOCAL, 1), (dict(b=1, L=4096, H=16), GLOBAL, 4), (dict(b=2, L=2048, H=8, init=True), LOCAL, 2),
+             (dict(P=128, H=4, G=2, L=1280), LOCAL, 4), (dict(b=1, L=4096, H=16), LOCAL, 4), (dict(L=2304, H=8), GLOBAL, 4)]
+    ws = torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda")
+    epoch = 0
+    for i, (kw, kernel, r) in enumerate(cases * 2):
+        d = oracle.make_inputs(3 if "nseq" in kw else 2, **kw)
+        want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"],
+                                              seq_idx=d["seq_idx"])
+        print(f"[epochs {i}] {kw} kernel={kernel} chunks/item={r} epoch={epoch}", flush=True)
+        out, fin = ops._fused_chunk_state_state_passing_fwd(
+            *[_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")], torch.float32, initial_states=_dev(d["initial_states"]),
+            seq_idx=_dev(d["seq_idx"]), _kernel=kernel, _chunks_per_item=r, _workspace=ws, _epoch=epoch)
+        assert ops._fused_workspace_status(ws) == 0
+        assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0, (i, kw)
+        epoch = 2 if epoch == 0 else epoch + 1
+    # a wait that runs out is reported for its own launch only, and the epochs go on
+    d = oracle.make_inputs(2, b=1, L=4096, H=16)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=GLOBAL, _chunks_per_item=1, _workspace=ws,
+                                             _epoch=epoch, _spin_limit=1)
+    assert ops._fused_workspace_status(ws) == -7
+    out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=GLOBAL, _chunks_per_item=1, _workspace=ws,
+                                                        _epoch=epoch + 1)
+    assert ops._fused_workspace_status(ws) == 0
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+def test_wrapper_keeps_its_own_workspace(ops, oracle):
+    # without a workspace argument the wrapper uses one of its own per (device, stream) and advances its epoch only when
+    # the chain kernel served the call: shapes that go to other kernel families in between must not disturb it
+    shapes = [dict(b=1, L=8192, H=80), dict(b=2, L=2048, H=8), dict(b=4, L=2048, H=80), dict(b=1, L=8192, H=80),
+              dict(b=3, L=4096, H=80), dict(b=2, L=2048, H=80), dict(b=1, L=8192, H=80)]
+    wants = {}
+    for rep in range(2):
+        for i, kw in enumerate(shapes):
+            d = oracle.make_inputs(2, **kw)
+            key = str(kw)
+            if key not in wants:
+                wants[key] = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+            out, fin = ops._fused_chunk_state_state_passing_fwd(*[_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")], torch.float32,
+                                                                initial_states=_dev(d["initial_states"]))
+            torch.cuda.synchronize()
+            assert _mismatches(out, wants[key][0])[0] == 0 and _mismatches(fin, wants[key][1])[0] == 0, (rep, i, kw)
+    # and on a second stream, with a workspace of its own
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    d = oracle.make_inputs(2, b=1, L=8192, H=80)
+    with torch.cuda.stream(st):
+        for _ in range(3):
+            out, fin = ops._fused_chunk_state_state_passing_fwd(*[_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")], torch.float32,
+                                                                initial_states=_dev(d["initial_states"]))
+    st.synchronize()
+    key = str(dict(b=1, L=8192, H=80))
+    assert _mismatches(out, wants[key][0])[0] == 0 and _mismatches(fin, wants[key][1])[0] == 0

@@ -49,7 +49,7 @@ def test_static_scratch_entry_point_two_calls(oracle):
 def test_static_scratch_rejects_what_does_not_fit():
     from ssd_amd import _lib
     lib = _lib.load()
-    # 262 144 ints: the header (64) plus one flag per (state tile, chunk).  b=8 L=131072 H=128 would need 1 M of them.
+    # 262 144 ints: the header (128) plus one flag per (state tile, chunk).  b=8 L=131072 H=128 would need 1 M of them.
     # The call is rejected before anything is launched, so the tensors only need plausible descriptions.
     b, L, H, P, N, G, Q, C = 8, 131072, 128, 64, 128, 8, 256, 512
     dims = _lib.dims_arg(b, L, H, P, N, G, Q, C)
