@@ -41,6 +41,8 @@ def test_struct_layouts_match_header():
     from ssd_amd import _lib
     assert ctypes.sizeof(_lib.SsdTensor) == 8 + 4 + 4 + 5 * 8
     assert ctypes.sizeof(_lib.SsdDims) == 8 * 4
+    assert ctypes.sizeof(_lib.SsdFusedOpts) == 8 + 8 + 4 * 4 + 8           # workspace, bytes, four ints, used_workspace
+    assert ctypes.sizeof(_lib.SsdFusedPlan) == 4 + 4 + 5 * 4
 
 
 def test_status_strings_and_argument_rejection_without_gpu(lib):
