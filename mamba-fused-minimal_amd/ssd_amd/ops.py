@@ -426,10 +426,9 @@ def set_segment_chunks(chunks):
 def set_token_split(waves):
     """Tuning / test hook (no counterpart in the reference): 2 or 4 = the token-split bf16 MFMA kernels with that
     many waves per state tile, 1 = the kernel with one wave per tile and four tiles per workgroup wherever it
-    applies, 3 = the kernel with three tiles per workgroup and the steps of a chunk dealt to the waves (fused call,
-    dstate 128, chunk 256, fp32 states; never chosen by the library itself), 0 = let the library choose.  Returns the
-    previous setting."""
+    applies, 0 = let the library choose.  While it is not 0 the library does not pick the ticket / flag-chain kernel by
+    itself either.  Returns the previous setting."""
     rc = _lib.load().ssd_set_token_split(int(waves))
     if rc < 0:
-        raise ValueError("token split must be 0, 1, 2, 3 or 4")
+        raise ValueError("token split must be 0, 1, 2 or 4")
     return rc
