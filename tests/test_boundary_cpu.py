@@ -204,3 +204,18 @@ def test_product_code_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header must compile as C99 (and as C++) on its own
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "ssd_gfx950.h"\n'
+                   "int main(void) { ssd_fused_opts o = {0}; ssd_fused_plan p; ssd_dims d = {0}; (void)o; (void)p; (void)d;\n"
+                   "  return SSD_FAMILY_COUNT == 5 && SSD_KERNEL_CHAIN_GLOBAL == 3 ? 0 : 1; }\n")
+    inc = os.path.join(ROOT, "include")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(src)], check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)], check=True)
