@@ -27,22 +27,53 @@ _WORKSPACES = {}
 _WORKSPACES_LOCK = threading.Lock()
 
 
+class _Epochs:
+    """The epochs of one kept workspace as ssd_fused_opts.epoch wants them: 0 for the first call (the library clears the
+    workspace and counts the call as epoch 1), then 2, 3, ... -- but only calls that ran the chain kernel count, a failed
+    call makes the contents unknown again, and the count starts over before it could overflow."""
+    LIMIT = 1 << 30
+
+    def __init__(self):
+        self.last = 0                      # epoch of the last chain launch on the workspace; 0 = contents unknown
+
+    def next(self):
+        if self.last >= self.LIMIT:
+            self.last = 0
+        return 0 if self.last == 0 else self.last + 1
+
+    def done(self, epoch, rc, used_workspace):
+        if rc:
+            self.last = 0
+        elif used_workspace:
+            self.last = max(epoch, 1)
+
+
 def _own_workspace(x, nbytes):
-    """-> (int32 tensor, epoch to pass).  Call with _WORKSPACES_LOCK held, and keep it until the launch is enqueued:
-    the epochs must reach the stream in order."""
+    """-> (int32 tensor, its _Epochs or None).  Call with _WORKSPACES_LOCK held, and keep it until the launch is
+    enqueued: the epochs must reach the stream in order."""
     stream = torch.cuda.current_stream(x.device)
     if torch.cuda.is_current_stream_capturing():
         # a captured launch is replayed with the same arguments: the same epoch again and again would take the flags of
         # the replay before for its own.  Epoch 0 (clear every time) is what a graph needs.
-        return torch.empty(((nbytes + 3) // 4,), device=x.device, dtype=torch.int32), 0
+        return torch.empty(((nbytes + 3) // 4,), device=x.device, dtype=torch.int32), None
     key = (x.device.index, stream.cuda_stream)
     ent = _WORKSPACES.get(key)
     if ent is None or ent[0].numel() * 4 < nbytes:
-        ent = [torch.empty((max(nbytes, 1 << 16) + 3) // 4, device=x.device, dtype=torch.int32), 0]
+        ent = (torch.empty((max(nbytes, 1 << 16) + 3) // 4, device=x.device, dtype=torch.int32), _Epochs())
         _WORKSPACES[key] = ent
-    ent[1] = 0 if ent[1] >= (1 << 30) else ent[1]
-    epoch = 0 if ent[1] == 0 else ent[1] + 1
-    return ent, epoch
+    return ent
+
+
+def _launch_on_own_workspace(x, nbytes, launch, used):
+    """Runs launch(workspace, epoch) -> status on the wrappers' workspace for x's device and stream."""
+    with _WORKSPACES_LOCK:
+        workspace, epochs = _own_workspace(x, nbytes)
+        if epochs is None:
+            return launch(workspace, 0)
+        epoch = epochs.next()
+        rc = launch(workspace, epoch)
+        epochs.done(epoch, rc, used.value)
+        return rc
 
 
 def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
@@ -187,16 +218,7 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     if _workspace is not None:
         rc = launch(_workspace, _epoch)
     else:
-        with _WORKSPACES_LOCK:
-            ent, epoch = _own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)))
-            if isinstance(ent, list):
-                rc = launch(ent[0], epoch)
-                if rc:
-                    ent[1] = 0                            # after a failed call the contents count as unknown
-                elif used.value:
-                    ent[1] = max(epoch, 1)                # only a call that ran the chain kernel used the epoch
-            else:
-                rc = launch(ent, 0)
+        rc = _launch_on_own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
     _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states
 
@@ -350,16 +372,7 @@ def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dty
     if _workspace is not None:
         rc = launch(_workspace, 0)
     else:
-        with _WORKSPACES_LOCK:
-            ent, epoch = _own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)))
-            if isinstance(ent, list):
-                rc = launch(ent[0], epoch)
-                if rc:
-                    ent[1] = 0
-                elif used.value:
-                    ent[1] = max(epoch, 1)
-            else:
-                rc = launch(ent, 0)
+        rc = _launch_on_own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
     _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd_ws")
     return out, final_states, dA_cumsum, dt_out
 

@@ -219,3 +219,25 @@ def test_header_is_plain_c(tmp_path):
     inc = os.path.join(ROOT, "include")
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(src)], check=True)
     subprocess.run(["g++", "-std=c++11", "-Wall", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)], check=True)
+
+
+def test_epochs_of_a_kept_workspace():
+    # what the wrappers pass as ssd_fused_opts.epoch for the workspace they keep per device and stream
+    from ssd_amd.ops import _Epochs
+    e = _Epochs()
+    assert e.next() == 0                                   # contents unknown: the library clears, the call counts as 1
+    e.done(0, 0, 1)
+    assert e.next() == 2
+    e.done(2, 0, 1)
+    assert e.next() == 3
+    e.done(3, 0, 0)                                        # another kernel family served the call: the epoch was not used
+    assert e.next() == 3
+    e.done(3, 0, 1)
+    assert e.next() == 4
+    e.done(4, -6, 0)                                       # a failed call: contents unknown again
+    assert e.next() == 0
+    e.done(0, 0, 0)                                        # cleared by nobody (not the chain kernel): still unknown
+    assert e.next() == 0
+    e.done(0, 0, 1)
+    e.last = _Epochs.LIMIT                                 # before the count could overflow it starts over
+    assert e.next() == 0
