@@ -14,7 +14,9 @@ The timed region is exactly K steps between two synchronisations.
 
 Besides the headline workload the line carries `per_config`: the fused call timed the same way on each of the five
 benchmark configurations (microseconds, GB/s of algorithmic bytes, fraction of HBM peak, TFLOP/s, parity mismatches
-against the CPU oracle).
+against the CPU oracle).  `roofline.plain_copy_gbps` is what a device-to-device copy of the same number of bytes (half
+read, half written) reaches in the same run, timed the same way, and `roofline.frac_of_plain_copy` the fused call's
+rate as a fraction of it: the published peak is not reachable by any kernel that reads and writes.
 """
 import argparse
 import json
@@ -183,6 +185,17 @@ def main():
         return ssd_amd._chunk_scan_states_fwd(C_dev[i % nsets], prev_states[i % nsets], s["dA_cumsum"], seq_idx=s["seq_idx"],
                                               out=y_bufs[i % nsets])
 
+    # what the part's memory system gives a kernel with nothing else to do: a device-to-device copy that reads half of
+    # the path's algorithmic bytes and writes the other half (the path reads x and writes `out`, about as much)
+    half = ssd_oracle.algorithmic_bytes(cfg, with_states=args.with_states) // 2
+    cp_src = [torch.empty(half, dtype=torch.uint8, device=dev).random_() for _ in range(nsets)]
+    cp_dst = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(nsets)]
+
+    def plain_copy(i):
+        cp_dst[i % nsets].copy_(cp_src[i % nsets])
+
+    _, copy_ev = timed(plain_copy, max(5, args.steps // 4), 3)
+    del cp_src, cp_dst
     _, bf16_ev = timed(fused_bf16, max(5, args.steps // 4), 3)
     _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
     _, prep_ev = timed(prep_fused, max(5, args.steps // 4), 3)
@@ -240,7 +253,9 @@ def main():
                      "traffic": None if args.with_states else measured_traffic(cfg["name"]),
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel sources with hash "
                                        + kernel_source_hash() + " (null: not measured on these sources)",
-                     "algorithmic_bytes": alg_bytes, "kernel_us": round(ev_step * 1e6, 2)},
+                     "algorithmic_bytes": alg_bytes, "kernel_us": round(ev_step * 1e6, 2),
+                     "plain_copy_us": round(copy_ev * 1e6, 2), "plain_copy_gbps": round(2 * half / copy_ev / 1e9, 1),
+                     "frac_of_plain_copy": round(copy_ev * 2 * half / alg_bytes / ev_step, 4)},
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "unfused_us": round(unf_ev * 1e6, 2),
