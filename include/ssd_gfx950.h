@@ -137,12 +137,14 @@ int ssd_fused_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, 
  * are resident.  The wait is bounded nevertheless (spin_limit polls): a wave that gives up sets the error word of the
  * workspace and still raises its own flag, so the launch always drains; ssd_fused_workspace_status reports it.
  *
- * workspace: device memory, 4-byte aligned, at least ssd_fused_workspace_bytes(dims); the call clears what it uses
+ * workspace: device memory, 4-byte aligned, at least ssd_fused_workspace_bytes(dims) -- with bf16 `out`: 16-byte
+ * aligned and at least ssd_fused_workspace_bytes_for(dims, SSD_BF16, chunks_per_item), see below --; the call clears what it uses
  * (a small fill launch, no memset node), so the memory may hold anything and may be reused by later calls on the
  * same stream (a caller that keeps a workspace to itself can save the fill launch: `epoch` below).  Two calls whose kernels may overlap (different streams) need workspaces of their own.
  * kernel: SSD_KERNEL_AUTO lets the library choose between this kernel and those of ssd_fused_chunk_state_passing_fwd
- * (which it runs when the shape, element types or a `states` output rule the chain kernel out: it needs bf16 x / B,
- * fp32 out / initial / final states, no `states`, dstate 64 or 128, chunk 128 or 256); SSD_KERNEL_CHAIN insists on it
+ * (which it runs when the shape, element types, a `states` output or too small a workspace rule the chain kernel out:
+ * it needs bf16 x / B, fp32 initial / final states, fp32 or bf16 out, no `states`, dstate 64 or 128, chunk 128 or
+ * 256); SSD_KERNEL_CHAIN insists on it
  * and returns SSD_ERR_SCRATCH where it cannot run; SSD_KERNEL_CHAIN_LOCAL / _GLOBAL also fix how passed states cross
  * between compute units, which the library otherwise chooses from the number of units per XCD (LOCAL: one ticket
  * counter per XCD over that XCD's share of the units, states exchanged through its L2; GLOBAL: one counter, states
@@ -169,6 +171,17 @@ typedef struct ssd_fused_opts {
 enum { SSD_KERNEL_AUTO = 0, SSD_KERNEL_CHAIN = 1, SSD_KERNEL_CHAIN_LOCAL = 2, SSD_KERNEL_CHAIN_GLOBAL = 3 };
 
 uint64_t ssd_fused_workspace_bytes(const ssd_dims *dims);
+/*
+ * The same for a given element type of `out`.  The reference's state passing keeps the running state in fp32
+ * registers over the whole sequence whatever `out` is stored as (kernels/ssd_state_passing.py:61-84); the chain
+ * kernel hands it from work item to work item through memory, so with bf16 `out` every item's last state is also
+ * written in fp32 to the workspace, where the next item reads it: 32 x dstate x 4 bytes per (state tile, item)
+ * behind the flags, i.e. 1 / chunks_per_item of an fp32 `out`.  chunks_per_item: the value the call will be given in
+ * ssd_fused_opts (0 = the library's choice for these sizes on the current device; with bf16 `out` items of one chunk
+ * are not offered).  Returns 0 where the chain kernel does not take that type (fp16 `out`, chunks_per_item == 1 with
+ * bf16): such calls run on the other kernels and need no workspace.  SSD_F32: ssd_fused_workspace_bytes(dims).
+ */
+uint64_t ssd_fused_workspace_bytes_for(const ssd_dims *dims, int out_dtype, int chunks_per_item);
 
 int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
                                          const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,

@@ -290,8 +290,15 @@ int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *
     if (opts && opts->used_workspace) *opts->used_workspace = 0;
     const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
     if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
-    const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % 4) == 0 &&
-                         opts->workspace_bytes >= ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+    // bf16 out: the workspace also holds the fp32 states that cross between items, as many as the launch will have
+    // items (the forced number of chunks per item, or the one the launch would choose)
+    const bool out16 = p.dt_out != ssd::DT_F32;
+    const int forced_r = opts ? opts->chunks_per_item : 0;
+    const int r = out16 ? ssd::chain_chunks_per_item(p, compute_units(), forced_r) : 0;
+    const uint64_t need = out16 ? ssd::chain_workspace_bytes_out16(dims->batch, dims->nheads, dims->headdim, dims->dstate, dims->nchunks, r)
+                                : ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+    const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % (out16 ? 16 : 4)) == 0 &&
+                         opts->workspace_bytes >= need && !(out16 && r < 2);
     if (have_ws && ssd::chain_supported(p) &&
         (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
         *use = true;
@@ -415,6 +422,20 @@ uint64_t ssd_fused_workspace_bytes(const ssd_dims *dims)
     return ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
 }
 
+uint64_t ssd_fused_workspace_bytes_for(const ssd_dims *dims, int out_dtype, int chunks_per_item)
+{
+    if (check_dims(dims)) return 0;
+    if (out_dtype == SSD_F32) return ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+    if (out_dtype != SSD_BF16) return 0;
+    Params p;
+    memset(&p, 0, sizeof(p));
+    p.batch = dims->batch; p.nheads = dims->nheads; p.headdim = dims->headdim; p.dstate = dims->dstate;
+    p.C = dims->nchunks; p.Q = dims->chunk_size; p.dt_out = ssd::DT_BF16;
+    const int r = ssd::chain_chunks_per_item(p, compute_units(), chunks_per_item);
+    if (r < 2) return 0;
+    return ssd::chain_workspace_bytes_out16(dims->batch, dims->nheads, dims->headdim, dims->dstate, dims->nchunks, r);
+}
+
 int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
                                          const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
                                          const ssd_tensor *initial_states, const ssd_tensor *states,
@@ -439,7 +460,9 @@ int ssd_fused_chunk_state_passing_fwd_static(const ssd_tensor *x, const ssd_tens
     Params p;
     int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, nullptr, out, final_states, dims, clamp);
     if (rc) return rc;
-    if (!ssd::chain_supported(p)) return SSD_ERR_SHAPE;        // only the kernel that needs scratch is offered here
+    // only the kernel that needs scratch is offered here, and its fp32 `out` only (the scratch has no room for the
+    // states that bf16 `out` makes it keep in fp32 as well)
+    if (!ssd::chain_supported(p) || p.dt_out != ssd::DT_F32) return SSD_ERR_SHAPE;
     if (ssd_fused_workspace_bytes(dims) > sizeof(int) * (uint64_t)kStaticScratchInts) return SSD_ERR_SCRATCH;
     rc = check_device();
     if (rc) return rc;

@@ -69,8 +69,12 @@ constexpr int kMaxXcd = 16;
 constexpr int kWsHeaderInts = kChainWsHeaderInts, kWsOwner = kChainWsOwnerWord;
 
 // NT = dstate / 16 (4 or 8); SPC = 32-token steps per chunk (4 or 8); R = chunks per work item (1, 2 or 4).
-// out, initial_states and final_states are fp32.
-template <int NT, int SPC, int R, bool HAS_SEQ, bool LOCAL>
+// initial_states and final_states are fp32; out is fp32, or (OUT16) bf16.  With bf16 passed states the state that
+// crosses from one item to the next must not be the rounded one -- the reference carries it in fp32 registers over
+// the whole sequence (kernels/ssd_state_passing.py:61-84) --, so an item's last state goes to memory twice: rounded
+// into out, and in fp32 into a slot of the workspace (p.carry: one 32 x dstate slot per tile and item), which is what
+// the next item reads back.  Per launch that is 1 / R of an fp32 `out` written and read on top of the bf16 one.
+template <int NT, int SPC, int R, bool HAS_SEQ, bool LOCAL, bool OUT16>
 __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 {
     constexpr int Q = 32 * SPC;
@@ -348,21 +352,40 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         const int64_t slice_out = (int64_t)(p.headdim - 1) * p.so_p + p.dstate;
         const int64_t slice_fin = (int64_t)(p.headdim - 1) * p.sf_p + p.dstate;
         const int64_t slice_in = (int64_t)(p.headdim - 1) * p.sin_p + p.dstate;
-        const float *outb = (const float *)p.out + I.b * p.so_b + I.h * p.so_h;
+        using out_t = std::conditional_t<OUT16, uint16_t, float>;
+        constexpr int kOutBytes = sizeof(out_t);
+        const out_t *outb = (const out_t *)p.out + I.b * p.so_b + I.h * p.so_h;
+        // the fp32 slot of (tile, item g) holds the state entering that item's first chunk g * R
+        constexpr int kSlotBytes = 32 * NT * 16 * 4;
+        auto carry_slot = [&](int c) { return make_rsrc((const char *)p.carry + ((int64_t)I.tile * n_super + c / R) * kSlotBytes, kSlotBytes); };
         const __amdgpu_buffer_rsrc_t rs_prev =
-            c0 > 0 ? make_rsrc(outb + (int64_t)c0 * p.so_c, slice_out * 4)
+            c0 > 0 ? (OUT16 ? carry_slot(c0) : make_rsrc(outb + (int64_t)c0 * p.so_c, slice_out * 4))
                    : make_rsrc((const float *)p.init + I.b * p.sin_b + I.h * p.sin_h, p.init ? slice_in * 4 : 0);
-        const int pitch_prev = c0 > 0 ? (int)p.so_p : (int)p.sin_p;
+        const int pitch_prev = c0 > 0 ? (OUT16 ? NT * 16 : (int)p.so_p) : (int)p.sin_p;
         const int row = I.p0 + 2 * (lane >> 2), col = 4 * (lane & 3);
+        const int row_prev = OUT16 && c0 > 0 ? 2 * (lane >> 2) : row;      // a slot holds the tile's 32 rows only
         int *const flag = ws_flags + (int64_t)I.tile * C;
         // chunk j of the item ends in out[:, c0 + j + 1], the sequence's last chunk in final_states
         auto store_chunk = [&](int j, const f32x4 (&v)[2 * NT], int aux) {
             const bool fin = c0 + j + 1 == C;
             const __amdgpu_buffer_rsrc_t rs = fin ? make_rsrc(p.fin + I.b * p.sf_b + I.h * p.sf_h, slice_fin * 4)
-                                                  : make_rsrc(outb + (int64_t)(c0 + j + 1) * p.so_c, slice_out * 4);
+                                                  : make_rsrc(outb + (int64_t)(c0 + j + 1) * p.so_c, slice_out * kOutBytes);
             const int pitch = fin ? (int)p.sf_p : (int)p.so_p;
+            if (OUT16 && !fin) {
+                // nobody reads these back inside the launch: plain stores whatever the mode
 #pragma unroll
-            for (int k = 0; k < 2 * NT; ++k) store4_f32(rs, row * pitch + col, (k & 1) * pitch + 16 * (k >> 1), v[k], aux);
+                for (int k = 0; k < 2 * NT; ++k) store4_bf16(rs, row * pitch + col, (k & 1) * pitch + 16 * (k >> 1), v[k]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 2 * NT; ++k) store4_f32(rs, row * pitch + col, (k & 1) * pitch + 16 * (k >> 1), v[k], aux);
+            }
+        };
+        // the item's last state in fp32, for the item behind it (OUT16 only)
+        auto store_carry = [&](int c_next, const f32x4 (&v)[2 * NT]) {
+            const __amdgpu_buffer_rsrc_t rs = carry_slot(c_next);
+#pragma unroll
+            for (int k = 0; k < 2 * NT; ++k)
+                store4_f32(rs, 2 * (lane >> 2) * (NT * 16) + col, (k & 1) * (NT * 16) + 16 * (k >> 1), v[k], kAux);
         };
 
         // held[j] <- exp(dA_j) [same sequence] held[j - 1] + held[j] for the chunks jb < j < je
@@ -387,7 +410,10 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         auto hand_on = [&]() {
             static_for<R>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                if (j == n - 1) store_chunk(j, held[j], kAux);
+                if (j == n - 1) {
+                    if (OUT16 && c0 + n < C) store_carry(c0 + n, held[j]);
+                    store_chunk(j, held[j], kAux);
+                }
             });
             if (c0 + n < C) {
                 asm volatile("" ::: "memory");
@@ -432,7 +458,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 s[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 if (read)
                     s[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                         rs_prev, 4 * (row * pitch_prev + col),
+                                                         rs_prev, 4 * (row_prev * pitch_prev + col),
                                                          4 * ((k & 1) * pitch_prev + 16 * (k >> 1)), kAux));
             }
             if (use_prev) {
@@ -445,8 +471,10 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             }
             if (c0 == 0) {
 #pragma unroll
-                for (int k = 0; k < 2 * NT; ++k)
-                    store4_f32(make_rsrc(outb, slice_out * 4), row * (int)p.so_p + col, (k & 1) * (int)p.so_p + 16 * (k >> 1), s[k], 0);
+                for (int k = 0; k < 2 * NT; ++k) {
+                    if (OUT16) store4_bf16(make_rsrc(outb, slice_out * 2), row * (int)p.so_p + col, (k & 1) * (int)p.so_p + 16 * (k >> 1), s[k]);
+                    else store4_f32(make_rsrc(outb, slice_out * 4), row * (int)p.so_p + col, (k & 1) * (int)p.so_p + 16 * (k >> 1), s[k], 0);
+                }
             }
         }
         // ... and runs through its chunks, in place: held[j] becomes the state after chunk c0 + j (an item that starts
@@ -666,13 +694,41 @@ size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks)
     return (size_t)(chain::kWsHeaderInts + tiles * nchunks) * sizeof(int);
 }
 
-// fp32 out / initial_states / final_states, no `states` output, and what the four-tile kernel asks of the inputs
+// ints in front of the fp32 carry slots: header and flags, rounded up to 256 bytes
+static int64_t carry_offset_ints(int64_t tiles, int nchunks)
+{
+    return (chain::kWsHeaderInts + tiles * nchunks + 63) / 64 * 64;
+}
+
+size_t chain_workspace_bytes_out16(int batch, int nheads, int headdim, int dstate, int nchunks, int chunks_per_item)
+{
+    const int64_t tiles = (int64_t)batch * nheads * ((headdim + 31) / 32);
+    const int r = chunks_per_item > 0 ? chunks_per_item : 1;
+    const int64_t items = (nchunks + r - 1) / r;
+    return (size_t)(carry_offset_ints(tiles, nchunks) * (int64_t)sizeof(int) + tiles * items * 32 * dstate * (int64_t)sizeof(float));
+}
+
+// Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units end up
+// with too few or too unequal numbers of items that large.  With bf16 `out` at least two: with one, the fp32 copies
+// of the passed states would be a whole fp32 `out`.
+int chain_chunks_per_item(const Params &p, int n_cu, int forced)
+{
+    if (forced == 1 || forced == 2 || forced == 4) return forced;
+    cost::Problem q;
+    q.units = (p.batch * p.nheads * (p.headdim / 32)) >> 2; q.chunks = p.C; q.chunk_size = p.Q; q.dstate = p.dstate;
+    q.n_cu = n_cu > 0 ? n_cu : 256;
+    const int r = cost::chain_chunks_per_item(q, nullptr);
+    return p.dt_out != DT_F32 && r < 2 ? 2 : r;
+}
+
+// fp32 initial_states / final_states, fp32 or bf16 out, no `states` output, and what the four-tile kernel asks of the
+// inputs
 bool chain_supported(const Params &p)
 {
     using namespace chain;
     if (p.states || !p.out || !p.fin) return false;
     if (!quad_inputs_supported(p)) return false;
-    if (p.dt_out != DT_F32 || (p.init && p.dt_init != DT_F32)) return false;
+    if ((p.dt_out != DT_F32 && p.dt_out != DT_BF16) || (p.init && p.dt_init != DT_F32)) return false;
     if (!rows_ok(p.out, p.so_b | p.so_c | p.so_h | p.so_p, p.so_p, p.headdim)) return false;
     if (!rows_ok(p.fin, p.sf_b | p.sf_h | p.sf_p, p.sf_p, p.headdim)) return false;
     if (p.init && !rows_ok(p.init, p.sin_b | p.sin_h | p.sin_p, p.sin_p, p.headdim)) return false;
@@ -680,36 +736,42 @@ bool chain_supported(const Params &p)
     return true;
 }
 
-template <int NT, int SPC, int R, bool SEQ, bool LOCAL>
+template <int NT, int SPC, int R, bool SEQ, bool LOCAL, bool OUT16>
 static hipError_t launch_chain_k(const Params &p, int n_wg, hipStream_t s)
 {
     constexpr int lds = chain::lds_bytes<NT, SPC>();
     static std::atomic<uint64_t> configured{0};
-    const hipError_t e = ensure_dynamic_lds((const void *)chain::chain_kernel<NT, SPC, R, SEQ, LOCAL>, lds, configured);
+    const hipError_t e = ensure_dynamic_lds((const void *)chain::chain_kernel<NT, SPC, R, SEQ, LOCAL, OUT16>, lds, configured);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((chain::chain_kernel<NT, SPC, R, SEQ, LOCAL>), dim3(n_wg), dim3(256), lds, s, p);
+    hipLaunchKernelGGL((chain::chain_kernel<NT, SPC, R, SEQ, LOCAL, OUT16>), dim3(n_wg), dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
-template <int R, bool SEQ, bool LOCAL>
+template <int R, bool SEQ, bool LOCAL, bool OUT16>
 static hipError_t launch_chain_r(const Params &p, int n_wg, hipStream_t s)
 {
     const int nt = p.dstate / 16, spc = p.Q / 32;
-    if (nt == 8 && spc == 8) return launch_chain_k<8, 8, R, SEQ, LOCAL>(p, n_wg, s);
-    if (nt == 8 && spc == 4) return launch_chain_k<8, 4, R, SEQ, LOCAL>(p, n_wg, s);
-    if (nt == 4 && spc == 8) return launch_chain_k<4, 8, R, SEQ, LOCAL>(p, n_wg, s);
-    return launch_chain_k<4, 4, R, SEQ, LOCAL>(p, n_wg, s);
+    if (nt == 8 && spc == 8) return launch_chain_k<8, 8, R, SEQ, LOCAL, OUT16>(p, n_wg, s);
+    if (nt == 8 && spc == 4) return launch_chain_k<8, 4, R, SEQ, LOCAL, OUT16>(p, n_wg, s);
+    if (nt == 4 && spc == 8) return launch_chain_k<4, 8, R, SEQ, LOCAL, OUT16>(p, n_wg, s);
+    return launch_chain_k<4, 4, R, SEQ, LOCAL, OUT16>(p, n_wg, s);
 }
 
 template <bool SEQ, bool LOCAL>
 static hipError_t launch_chain_t(const Params &p, int r, int n_wg, hipStream_t s)
 {
-    if (r >= 4) return launch_chain_r<4, SEQ, LOCAL>(p, n_wg, s);
-    if (r >= 2) return launch_chain_r<2, SEQ, LOCAL>(p, n_wg, s);
-    return launch_chain_r<1, SEQ, LOCAL>(p, n_wg, s);
+    if (p.dt_out != DT_F32) {       // bf16 out: items of one chunk are not offered (chain_chunks_per_item)
+        if (r >= 4) return launch_chain_r<4, SEQ, LOCAL, true>(p, n_wg, s);
+        return launch_chain_r<2, SEQ, LOCAL, true>(p, n_wg, s);
+    }
+    if (r >= 4) return launch_chain_r<4, SEQ, LOCAL, false>(p, n_wg, s);
+    if (r >= 2) return launch_chain_r<2, SEQ, LOCAL, false>(p, n_wg, s);
+    return launch_chain_r<1, SEQ, LOCAL, false>(p, n_wg, s);
 }
 
-// p.ws: at least chain_workspace_bytes(...) of device memory, 4-byte aligned; the launch clears what it uses.
+// p.ws: at least chain_workspace_bytes(...) of device memory, 4-byte aligned (bf16 out: chain_workspace_bytes_out16(...)
+// for the chunks per item that chain_chunks_per_item(p, n_cu, p.n_seg) gives, 16-byte aligned); the launch clears what
+// it uses.
 // n_cu: compute units of the device.  mode: 0 = choose, 1 = LOCAL, 2 = GLOBAL.
 hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
 {
@@ -742,11 +804,10 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     const bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
     // Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units
     // end up with too few or too unequal numbers of items that large.  p.n_seg > 0 forces a value.
-    int r = p.n_seg;
-    if (r <= 0) {
-        cost::Problem q;
-        q.units = n_units; q.chunks = p.C; q.chunk_size = p.Q; q.dstate = p.dstate; q.n_cu = n_cu > 0 ? n_cu : 256;
-        r = cost::chain_chunks_per_item(q, nullptr);
+    const int r = chain_chunks_per_item(p, n_cu, p.n_seg);
+    if (p.dt_out != DT_F32) {
+        if (r < 2) return hipErrorInvalidValue;
+        p.carry = (float *)(p.ws + carry_offset_ints(p.n_items, p.C));
     }
     const int64_t total = (int64_t)n_units * ((p.C + r - 1) / r);
     int n_wg = (int)(total < n_cu ? total : n_cu);

@@ -41,6 +41,7 @@ struct Params {
     int n_cu;             // compute units of the device (0: not known, the launchers then assume 256 in 8 XCDs)
     int ws_cleared;       // the launch in front of that kernel has cleared `ws` already (chain_workspace_clear below)
     int epoch;            // of this launch on `ws` (below); <= 0: contents unknown, the launcher clears it and takes 1
+    float *carry;         // inside `ws`, behind the flags: the fp32 states that cross between items when `out` is 16-bit
 };
 
 // State passing on a flattened state axis.
@@ -168,6 +169,9 @@ int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup o
 hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
 bool chain_supported(const Params &p);
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
+// ... and with room for the fp32 states that cross between items of `chunks_per_item` chunks when `out` is bf16
+size_t chain_workspace_bytes_out16(int batch, int nheads, int headdim, int dstate, int nchunks, int chunks_per_item);
+int chain_chunks_per_item(const Params &p, int n_cu, int forced);     // what launch_chain takes (forced: 0, 1, 2 or 4)
 
 // Layout of a chain workspace (ints).  A launch carries an epoch, one more than that of the launch before it on the
 // same workspace.  Everything a launch must find in a known state is either tagged with the epoch or kept twice:
@@ -179,6 +183,8 @@ size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
 //   [96 + slot]    hardware id (+1) of the XCD that drew from each slot
 //   [128 ...]      flags, one per (state tile, chunk): raised = holds the epoch of the launch (older values, from
 //                  launches before, and the zeros of a clearing never equal it)
+//   behind the flags, from the next multiple of 64 ints: 32 x dstate fp32 per (state tile, item) when `out` is bf16;
+//                  written before it is read in every launch, never cleared
 constexpr int kChainWsHeaderInts = 128, kChainWsBankStride = 32, kChainWsErrWord = 64, kChainWsEpochWord = 66,
               kChainWsTagWord = 67, kChainWsOwnerWord = 96, kChainWsTag = 0x53534443;
 // The value a cleared chain workspace holds at int i: zero, except for the tag.  Any kernel that runs in front of the

@@ -50,6 +50,14 @@ __device__ __forceinline__ void store4_f32(__amdgpu_buffer_rsrc_t rs, int voff, 
     asm volatile("s_nop 3" ::"v"(q) : "memory");
 }
 
+// The same four values rounded to bf16 (nearest even): 8 bytes, default cache policy.
+__device__ __forceinline__ void store4_bf16(__amdgpu_buffer_rsrc_t rs, int voff, int soff, f32x4 v)
+{
+    const u32x2 q = {pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+    __builtin_amdgcn_raw_buffer_store_b64(q, rs, 2 * voff, 2 * soff, 0);
+    asm volatile("s_nop 3" ::"v"(q) : "memory");
+}
+
 
 // Compile-time model of the vector-memory queue of the step loops that stream x and B through LDS rings
 // (ssd_quad.hip, ssd_chain.hip).  Per 32-token step t these kernels issue, in this program order,

@@ -13,7 +13,7 @@ SSD_F32, SSD_BF16, SSD_F16 = 0, 1, 2
 _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_F16}
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
-           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes",
+           "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes", "ssd_fused_workspace_bytes_for",
            "ssd_fused_workspace_status", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
            "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd_ws", "ssd_query_path", "ssd_query_fused_plan", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
@@ -68,6 +68,8 @@ def load():
     lib.ssd_fused_chunk_state_passing_fwd_ws.argtypes = [T, T, T, T, T, T, T, T, T, D, ctypes.c_int, ctypes.POINTER(SsdFusedOpts), vp]
     lib.ssd_fused_workspace_bytes.restype = ctypes.c_uint64
     lib.ssd_fused_workspace_bytes.argtypes = [D]
+    lib.ssd_fused_workspace_bytes_for.restype = ctypes.c_uint64
+    lib.ssd_fused_workspace_bytes_for.argtypes = [D, ctypes.c_int, ctypes.c_int]
     lib.ssd_fused_workspace_status.restype = ctypes.c_int
     lib.ssd_fused_workspace_status.argtypes = [vp, vp]
     lib.ssd_fused_chunk_state_passing_fwd_static.restype = ctypes.c_int

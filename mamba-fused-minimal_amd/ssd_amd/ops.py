@@ -169,7 +169,8 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
 
     The reference's wrappers allocate their counters per call (kernels/fused_globalbar.py:237-238,
     kernels/fused_concurrent.py:296-298); so does this one: a small int32 workspace for the ticket counter and the
-    flags of the kernel that spreads a sequence's chunks over all compute units.  ``_kernel`` (0 = let the library
+    flags of the kernel that spreads a sequence's chunks over all compute units (plus, with bf16 ``out_dtype``, the
+    fp32 copies of the states that cross between that kernel's work items).  ``_kernel`` (0 = let the library
     choose, 1 = insist on that kernel, 2 / 3 = and on its per-XCD / device-wide variant), ``_chunks_per_item``
     (1, 2 or 4 consecutive chunks per work item of that kernel, 0 = choose), ``_spin_limit`` (polls before a flag wait gives up, 0 = default) and
     ``_workspace`` (an int32 tensor to use instead of the wrapper's own, which it keeps per device and stream and whose
@@ -218,7 +219,10 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     if _workspace is not None:
         rc = launch(_workspace, _epoch)
     else:
-        rc = _launch_on_own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
+        # bf16 passed states: the workspace also takes the fp32 states that cross between work items (a quarter of
+        # an fp32 `out`, as a rule); 0 = that kernel is not offered for these arguments
+        nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out_dtype, -1), int(_chunks_per_item)))
+        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
     _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states
 
@@ -372,7 +376,8 @@ def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dty
     if _workspace is not None:
         rc = launch(_workspace, 0)
     else:
-        rc = _launch_on_own_workspace(x, int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
+        nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out.dtype, -1), int(_chunks_per_item)))
+        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
     _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd_ws")
     return out, final_states, dA_cumsum, dt_out
 

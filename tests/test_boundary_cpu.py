@@ -85,6 +85,25 @@ def test_status_strings_and_argument_rejection_without_gpu(lib):
     assert lib.ssd_set_segment_chunks(-1) == -2 and lib.ssd_set_segment_chunks(3) == 0 and lib.ssd_set_segment_chunks(0) == 3
 
 
+def test_workspace_size_by_element_type_of_the_passed_states(lib):
+    # fp32 `out`: header + a flag per (state tile, chunk).  bf16 `out`: that, rounded up to 256 bytes, and 32 x dstate
+    # fp32 per (state tile, work item) -- the running state crosses between work items in fp32, as the reference keeps
+    # it in registers (kernels/ssd_state_passing.py:61-84).  fp16 `out`, or bf16 with items of one chunk: not offered.
+    from ssd_amd import _lib
+    big = _lib.dims_arg(4, 8192, 80, 64, 128, 1, 256, 32)
+    tiles, flags = 4 * 80 * 2, 128 + 4 * 80 * 2 * 32
+    assert lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_F32, 0) == lib.ssd_fused_workspace_bytes(big) == 4 * flags
+    for r in (2, 4):
+        want = 4 * ((flags + 63) // 64 * 64) + tiles * (32 // r) * 32 * 128 * 4
+        assert lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_BF16, r) == want
+    assert lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_BF16, 0) == lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_BF16, 4)
+    assert lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_BF16, 1) == 0
+    assert lib.ssd_fused_workspace_bytes_for(big, _lib.SSD_F16, 0) == 0
+    odd = _lib.dims_arg(1, 2304, 8, 64, 128, 1, 256, 9)                # 9 chunks: 5 items of two, 3 of four
+    assert lib.ssd_fused_workspace_bytes_for(odd, _lib.SSD_BF16, 2) == 4 * ((128 + 16 * 9 + 63) // 64 * 64) + 16 * 5 * 32 * 128 * 4
+    assert lib.ssd_fused_workspace_bytes_for(odd, _lib.SSD_BF16, 4) == 4 * ((128 + 16 * 9 + 63) // 64 * 64) + 16 * 3 * 32 * 128 * 4
+
+
 def test_argument_validation_from_two_threads_with_different_hooks(lib):
     # The three ssd_set_* hooks are process-wide atomics and everything else is per call: two host threads that keep
     # setting different hook values while they call the argument-validation paths (which return before any device

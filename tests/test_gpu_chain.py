@@ -74,6 +74,56 @@ def test_chain_kernel_variants(ops, oracle, kw, kernel, r):
     _chain_case(ops, oracle, oracle.make_inputs(1, **base), kernel, r, f"chain.k{kernel}.r{r}")
 
 
+def _bf16_workspace_ints(x, B, dt, r):
+    # header + a flag per (state tile, chunk), rounded up to 256 bytes, then 32 x dstate fp32 per (state tile, item)
+    tiles, C, N = x.shape[0] * x.shape[2] * (x.shape[3] // 32), dt.shape[2], B.shape[-1]
+    return (128 + tiles * C + 63) // 64 * 64 + tiles * ((C + r - 1) // r) * 32 * N
+
+
+@pytest.mark.parametrize("r", [2, 4])
+@pytest.mark.parametrize("kernel", [LOCAL, GLOBAL], ids=["local", "global"])
+@pytest.mark.parametrize("kw", SHAPES + [dict(L=4096, H=8, nseq=6, init=True)], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_chain_bf16_passed_states(ops, oracle, kw, kernel, r):
+    # bf16 `out` (what the reference's main.py asks for, out_dtype = C.dtype): the state that crosses between work
+    # items stays fp32 (kernels/ssd_state_passing.py:61-84 keeps it in registers), through a slot of the workspace.  So
+    # the final states are those of the fp32 call bit for bit, and `out` is the fp32 call's `out` rounded once.
+    from ssd_amd import _lib
+    base = dict(b=2, L=1024, H=6, G=1)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    name = f"chain.bf16out.k{kernel}.r{r}"
+    out32, fin32 = _chain_case(ops, oracle, d, kernel, r, name + ".fp32")
+    x, B, dt, dAcs, seq, init = d["x"], d["B"], d["dt"], d["dA_cumsum"], d["seq_idx"], d["initial_states"]
+    n_ints = _bf16_workspace_ints(x, B, dt, r)
+    dims = _lib.dims_arg(x.shape[0], x.shape[1], x.shape[2], x.shape[3], B.shape[-1], B.shape[2], dt.shape[3], dt.shape[2])
+    assert int(_lib.load().ssd_fused_workspace_bytes_for(dims, _lib.SSD_BF16, r)) == 4 * n_ints
+    ws = torch.full((n_ints,), -1, dtype=torch.int32, device="cuda")           # garbage, the fp32 slots included
+    print(f"[{name}] x{tuple(x.shape)} workspace {4 * n_ints} bytes", flush=True)
+    out16, fin16 = ops._fused_chunk_state_state_passing_fwd(
+        _dev(B), _dev(x), _dev(dt), _dev(dAcs), torch.bfloat16, initial_states=_dev(init), seq_idx=_dev(seq),
+        _kernel=kernel, _chunks_per_item=r, _workspace=ws)
+    assert ops._fused_workspace_status(ws) == 0
+    assert out16.dtype == torch.bfloat16 and torch.isfinite(out16.float()).all()
+    assert torch.equal(fin16, fin32), f"{name}: final states differ, max {float((fin16 - fin32).abs().max()):.3e}"
+    assert torch.equal(out16, out32.to(torch.bfloat16)), f"{name}: out differs, max {float((out16.float() - out32).abs().max()):.3e}"
+
+
+def test_chain_bf16_passed_states_left_to_the_library(ops, oracle):
+    # no hooks: the wrapper sizes its own workspace for bf16 `out` and the library picks the kernel (32 chunks on 40
+    # units: the chain kernel); a second call reuses the workspace with the next epoch
+    d = oracle.make_inputs(2, b=1, L=8192, H=40)
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    for i in range(2):
+        out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, initial_states=_dev(d["initial_states"]))
+        torch.cuda.synchronize()
+        assert out.dtype == torch.bfloat16
+        bad, worst = _mismatches(out, want_out, rtol=RTOL + 2.0 ** -8)
+        assert bad == 0, f"call {i}: out {bad} mismatches, max {worst:.3e}"
+        bad, worst = _mismatches(fin, want_fin)
+        assert bad == 0, f"call {i}: final {bad} mismatches, max {worst:.3e}"
+
+
 @pytest.mark.parametrize("r", [2, 4])
 @pytest.mark.parametrize("kernel", [LOCAL, GLOBAL], ids=["local", "global"])
 def test_chain_items_cut_by_sequence_starts(ops, oracle, kernel, r):
@@ -207,8 +257,15 @@ def test_chain_rejections(ops, oracle):
     small = torch.zeros(8, dtype=torch.int32, device="cuda")
     with pytest.raises(RuntimeError, match="workspace"):                       # forced, workspace too small
         ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=1, _workspace=small)
-    with pytest.raises(RuntimeError, match="workspace"):                       # forced, 16-bit out is not its job
-        ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, _kernel=1)
+    with pytest.raises(RuntimeError, match="workspace"):                       # forced, fp16 out is not its job
+        ops._fused_chunk_state_state_passing_fwd(*args, torch.float16, _kernel=1)
+    with pytest.raises(RuntimeError, match="workspace"):                       # forced, bf16 out with items of one chunk
+        ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, _kernel=1, _chunks_per_item=1)
+    flags_only = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="workspace"):                       # forced, bf16 out, no room for the fp32 copies
+        ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, _kernel=1, _workspace=flags_only)
+    out16, _ = ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, _workspace=flags_only)      # not forced: another kernel
+    assert out16.dtype == torch.bfloat16
     # left to itself the library falls back to its other kernels in both situations
     out, fin = ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _workspace=small)
     want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
