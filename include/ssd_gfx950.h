@@ -205,7 +205,8 @@ int ssd_fused_workspace_status(const void *workspace, void *stream);
  * flags live in a fixed 1 MiB array inside the library's own code object (one copy per GPU, held until the process
  * ends); the call clears what it uses with a small fill launch and runs the chain kernel, whatever the problem size
  * (the kernel choice of the other entry points is not made here: SSD_ERR_SHAPE for arguments that kernel does not
- * cover -- it needs bf16 x / B, fp32 out / initial / final states, dstate 64 or 128, chunk 128 or 256 --,
+ * cover -- it needs bf16 x / B, fp32 out / initial / final states (bf16 out needs room the array does not have),
+ * dstate 64 or 128, chunk 128 or 256 --,
  * SSD_ERR_SCRATCH when batch * nheads * (headdim / 32) * nchunks + 128 ints do not fit the array, i.e. above 262 016
  * (state tile, chunk) pairs).  Every call on a GPU shares that GPU's array: two calls whose kernels may overlap
  * (different streams, different host threads) race on it and must be serialised by the caller.
