@@ -73,6 +73,15 @@ def test_static_scratch_rejects_what_does_not_fit():
         described(_lib.SSD_F32, (b, H, P, N)), dims, 1, None)
     assert rc == _lib.SSD_ERR_SCRATCH, rc
     assert "workspace" in lib.ssd_status_string(rc).decode()
+    # bf16 passed states: the chain kernel would keep fp32 copies of them in its workspace, for which the array has no
+    # room -- a shape this entry point does not cover, whatever the size
+    b, L, C = 1, 1024, 4
+    small = _lib.dims_arg(b, L, H, P, N, G, Q, C)
+    rc = lib.ssd_fused_chunk_state_passing_fwd_static(
+        described(_lib.SSD_BF16, (b, L, H, P)), described(_lib.SSD_BF16, (b, L, G, N)), described(_lib.SSD_F32, (b, H, C, Q)),
+        described(_lib.SSD_F32, (b, H, C, Q)), none, none, described(_lib.SSD_BF16, (b, C, H, P, N)),
+        described(_lib.SSD_F32, (b, H, P, N)), small, 1, None)
+    assert rc == -2, rc                      # SSD_ERR_SHAPE
 
 
 def test_static_entry_point_inside_a_hip_graph(oracle):
