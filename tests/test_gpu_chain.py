@@ -190,6 +190,19 @@ def test_dt_preparation_and_chain_kernel_in_one_call(ops, oracle, kw, kernel):
                                                               _workspace=torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda"))
         torch.cuda.synchronize()
         assert torch.equal(dt2, dt) and torch.equal(dA2, dA) and torch.equal(out2, out) and torch.equal(fin2, fin)
+    # the same call with bf16 passed states on the wrapper's own workspace: final states as above, `out` rounded once
+    out16, fin16, _, _ = ops._fused_cumsum_chunk_state_state_passing_fwd(
+        _dev(d["B"]), _dev(d["x"]), _dev(raw), _dev(A), Q, torch.bfloat16, dt_bias=_dev(bias), dt_softplus=True,
+        initial_states=_dev(init), seq_idx=_dev(seq), _kernel=kernel)
+    torch.cuda.synchronize()
+    assert out16.dtype == torch.bfloat16
+    if kernel != 0:                                        # same kernel, same chunks per item unless the library chose
+        bad, worst = _mismatches(fin16, fin.cpu(), 1e-5, 1e-6)
+        assert bad == 0, f"prep+chain.bf16.final: {bad} mismatches, max abs err {worst:.3e}"
+    bad, worst = _mismatches(out16, want_out, RTOL + 2.0 ** -8, ATOL)
+    assert bad == 0, f"prep+chain.bf16.out: {bad} mismatches, max abs err {worst:.3e}"
+    bad, worst = _mismatches(fin16, want_fin)
+    assert bad == 0, f"prep+chain.bf16.final: {bad} mismatches, max abs err {worst:.3e}"
 
 
 def test_chain_local_with_fewer_units_than_xcds(ops, oracle):
