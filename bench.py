@@ -200,6 +200,9 @@ def main():
     _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
     _, prep_ev = timed(prep_fused, max(5, args.steps // 4), 3)
     _, scan_ev = timed(scan_states, max(5, args.steps // 4), 3)
+    # ... and on bf16 passed states (the reference's main.py hands its scan `out` in C's type)
+    prev_states = [fused_bf16(i)[0] for i in range(nsets)]
+    _, scan16_ev = timed(scan_states, max(5, args.steps // 4), 3)
     del prev_states, y_bufs
 
     # parity of what was timed, over the whole batch, against the CPU oracle (the long grouped configuration on four
@@ -263,6 +266,7 @@ def main():
         "chunk_cumsum_us": round(cs_ev * 1e6, 2),
         "fused_with_dt_preparation_us": round(prep_ev * 1e6, 2),
         "chunk_scan_states_us": round(scan_ev * 1e6, 2),
+        "chunk_scan_states_from_bf16_us": round(scan16_ev * 1e6, 2),
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,
         "parity_scope": scope,
