@@ -64,6 +64,14 @@ def _own_workspace(x, nbytes):
     return ent
 
 
+def release_workspaces():
+    """Drops the workspaces the fused wrappers keep per (device, stream): a few hundred KB each as a rule, a quarter
+    of an fp32 ``out`` after a call with bf16 passed states.  The next call allocates (and clears) a new one.  Launches
+    already enqueued keep theirs alive through the caching allocator's stream ordering."""
+    with _WORKSPACES_LOCK:
+        _WORKSPACES.clear()
+
+
 def _launch_on_own_workspace(x, nbytes, launch, used):
     """Runs launch(workspace, epoch) -> status on the wrappers' workspace for x's device and stream."""
     with _WORKSPACES_LOCK:
@@ -221,7 +229,9 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
     else:
         # bf16 passed states: the workspace also takes the fp32 states that cross between work items (a quarter of
         # an fp32 `out`, as a rule); 0 = that kernel is not offered for these arguments
-        nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out_dtype, -1), int(_chunks_per_item)))
+        nbytes = 0
+        if states is None:          # with a `states` buffer the call runs on other kernels anyway
+            nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out_dtype, -1), int(_chunks_per_item)))
         rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
     _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states

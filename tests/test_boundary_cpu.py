@@ -240,6 +240,15 @@ def test_header_is_plain_c(tmp_path):
     subprocess.run(["g++", "-std=c++11", "-Wall", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)], check=True)
 
 
+def test_kept_workspaces_can_be_released():
+    import ssd_amd
+    from ssd_amd import ops
+    with ops._WORKSPACES_LOCK:
+        ops._WORKSPACES[("test", 0)] = (torch.zeros(4, dtype=torch.int32), ops._Epochs())
+    ssd_amd.release_workspaces()
+    assert not ops._WORKSPACES
+
+
 def test_epochs_of_a_kept_workspace():
     # what the wrappers pass as ssd_fused_opts.epoch for the workspace they keep per device and stream
     from ssd_amd.ops import _Epochs
