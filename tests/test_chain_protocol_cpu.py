@@ -12,7 +12,10 @@ promises nothing about residency.  Checked: every launch drains, every passed st
 (ssd_state_passing.py:69-84 on scalars), no wait gives up when the limit is generous, and a limit of one poll is
 reported while the launch still drains.  A workspace may be kept from launch to launch without clearing: flags hold the
 epoch they were raised in, ticket counters and error words exist once per parity of the epoch, and the workgroup that
-draws ticket 0 zeroes the other parity's for the launch after it (the last test)."""
+draws ticket 0 zeroes the other parity's for the launch after it.  With 16-bit passed states an item's last state is
+stored twice -- rounded into `out`, exact into a slot of the workspace that the next item reads instead of `out` -- and
+those slots are never cleared: the last test keeps a workspace full of stale slots and checks that the final states are
+those of the exact recurrence and `out` is that recurrence rounded once."""
 import random
 
 import pytest
@@ -28,6 +31,7 @@ class Workspace:
         self.errors = [0, 0]
         self.last_epoch = 0
         self.flags = [0] * n_flags
+        self.carry = [float("nan")] * n_flags      # exact copies of the states that cross between items; never cleared
 
     def status(self):
         return self.errors[self.last_epoch & 1]
@@ -48,7 +52,7 @@ class _Flags:
 
 
 class Launch:
-    def __init__(self, n_units, C, R, n_wg, resident, spin_limit, seed, boundaries=(), ws=None, epoch=1):
+    def __init__(self, n_units, C, R, n_wg, resident, spin_limit, seed, boundaries=(), ws=None, epoch=1, rounded=False):
         self.n_units, self.C, self.R, self.n_wg, self.resident, self.spin_limit = n_units, C, R, n_wg, resident, spin_limit
         self.rng = random.Random(seed)
         self.n_super = (C + R - 1) // R
@@ -63,6 +67,12 @@ class Launch:
         self.init = [self.rng.uniform(-1, 1) for _ in range(n_units)]
         self.out = [[None] * (C + 1) for _ in range(n_units)]       # out[u][c] = state entering chunk c; [C] = final
         self.events = 0
+        # rounded: `out` holds rounded states (16-bit passed states), the exact ones cross through self.ws.carry
+        self.rounded = rounded
+        self.rnd = (lambda v: round(v, 2)) if rounded else (lambda v: v)
+
+    def slot(self, u, c):
+        return u * self.n_super + c // self.R
 
     @property
     def ticket(self):
@@ -118,8 +128,13 @@ class Launch:
             jz = max([r for r in range(1, n) if scale[r] == 0.0], default=0)
 
             def hand_on():
-                self.out[u][c0 + n] = held[n - 1]
-                yield                                  # the store is acknowledged ...
+                if c0 + n < self.C:
+                    if self.rounded:
+                        self.ws.carry[self.slot(u, c0 + n)] = held[n - 1]
+                    self.out[u][c0 + n] = self.rnd(held[n - 1])
+                else:
+                    self.out[u][c0 + n] = held[n - 1]  # the final state is never rounded
+                yield                                  # the stores are acknowledged ...
                 if c0 + n < self.C:
                     self.flag[u][c0 + n] = 1           # ... before the flag goes up
 
@@ -137,16 +152,21 @@ class Launch:
                         break
                     yield
             if c0 == 0:
-                self.out[u][0] = self.init[u]
+                self.out[u][0] = self.rnd(self.init[u])
             if use_prev:
-                prev = self.out[u][c0] if self.out[u][c0] is not None else float("nan")   # gave up: whatever is there
+                if c0 == 0:
+                    prev = self.init[u]
+                elif self.rounded:
+                    prev = self.ws.carry[self.slot(u, c0)]                                  # gave up: whatever is there
+                else:
+                    prev = self.out[u][c0] if self.out[u][c0] is not None else float("nan")
                 held[0] += scale[0] * prev
             for r in range(1, jz if jz > 0 else n):
                 held[r] += scale[r] * held[r - 1]
             if jz == 0:
                 yield from hand_on()
             for r in range(n - 1):                     # the states inside the item
-                self.out[u][c0 + r + 1] = held[r]
+                self.out[u][c0 + r + 1] = self.rnd(held[r])
             yield
             cur, nxt, after, late = nxt, after, None, False
 
@@ -242,3 +262,24 @@ def test_a_workspace_kept_from_launch_to_launch_with_epochs():
                     assert abs(L.out[u][c] - want[u][c]) <= 1e-12 * max(1.0, abs(want[u][c])), (i, u, c)
         epoch += 1
     assert ws.tickets[epoch & 1] == 0            # the bank of the launch that would come next is clean
+
+
+def test_rounded_passed_states_cross_between_items_exactly():
+    # 16-bit `out`: the state entering an item is read from the workspace slot its predecessor wrote in this launch,
+    # never from the rounded `out` and never from what an earlier launch (other sizes, other slot mapping) left there
+    rng = random.Random(11)
+    ws = Workspace()
+    epoch = 1
+    for i in range(40):
+        n_units, C, R, n_wg = rng.choice([sh for sh in SHAPES if sh[2] > 1])
+        resident = rng.choice([1, 2, 3, 1000])
+        boundaries = {(rng.randrange(n_units), rng.randrange(C)) for _ in range((n_units * C) // 7)} if i % 2 else set()
+        L = Launch(n_units, C, R, n_wg, resident, spin_limit=1 << 30, seed=300 + i, boundaries=boundaries, ws=ws, epoch=epoch,
+                   rounded=i % 3 != 2).run()
+        assert ws.status() == 0, i
+        want = L.reference()
+        for u in range(n_units):
+            assert abs(L.out[u][C] - want[u][C]) <= 1e-12 * max(1.0, abs(want[u][C])), (i, u)
+            for c in range(C):
+                assert abs(L.out[u][c] - L.rnd(want[u][c])) <= (1e-2 + 1e-9 if L.rounded else 1e-12 * max(1.0, abs(want[u][c]))), (i, u, c)
+        epoch += 1
