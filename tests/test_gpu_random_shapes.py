@@ -60,6 +60,14 @@ def test_random_shape(ops, oracle, seed):
             err = (got - want).abs()
             bad = int((err > ATOL + RTOL * want.abs()).sum())
             assert bad == 0, f"seed {seed} {kw} {name}.{what}: {bad} mismatches, max abs err {float(err.max()):.3e}"
+    # the forced chain launch again with bf16 passed states, on the wrapper's own workspace: the running state crosses
+    # between work items in fp32, so the final states are the same bits and `out` is the fp32 `out` rounded once (the
+    # number of chunks per item does not change the arithmetic; with bf16 `out` it is at least two)
+    out16, fin16 = ops._fused_chunk_state_state_passing_fwd(*args, torch.bfloat16, initial_states=_dev(init), seq_idx=_dev(seq),
+                                                            _kernel=kernel, _chunks_per_item=max(r, 2))
+    torch.cuda.synchronize()
+    assert torch.equal(fin16, fin), f"seed {seed} {kw}: final states with bf16 out differ, max {float((fin16 - fin).abs().max()):.3e}"
+    assert torch.equal(out16, out.to(torch.bfloat16)), f"seed {seed} {kw}: bf16 out is not the fp32 out rounded"
 
 
 def _draw_any(seed):
