@@ -55,7 +55,11 @@ typedef enum ssd_status {
     SSD_ERR_STRIDE = -4,      /* innermost stride != 1 where the kernels need it */
     SSD_ERR_DEVICE = -5,      /* current device is not gfx950, or no device */
     SSD_ERR_SCRATCH = -6,     /* a kernel was asked for that needs a workspace, and none (or too small a one) was given */
-    SSD_ERR_CHAIN_TIMEOUT = -7 /* reported by ssd_fused_workspace_status: a bounded flag wait ran out */
+    /* reported by ssd_fused_workspace_status about the last launch of the ticket / flag-chain kernel (outputs unusable): */
+    SSD_ERR_CHAIN_TIMEOUT = -7,    /* a bounded flag wait ran out */
+    SSD_ERR_CHAIN_XCD = -8,        /* workgroups of two XCDs drew from one per-XCD ticket counter */
+    SSD_ERR_CHAIN_INCOMPLETE = -9, /* a ticket counter that owns work items was never served: their outputs were not written */
+    SSD_ERR_CHAIN_WORKSPACE = -10  /* the workspace was not what ssd_fused_opts.epoch promised */
 } ssd_status;
 
 /* A strided device tensor.  stride[i] is in elements; unused trailing entries are ignored. */
@@ -160,10 +164,15 @@ typedef struct ssd_fused_opts {
     int32_t epoch;            /* chain kernel: 0 = the workspace may hold anything, the call clears it with a small fill
                                  launch (default).  n > 0 = a promise that saves that launch: the call before this one on
                                  this workspace (same stream, or ordered before it) was made with epoch n - 1, or with
-                                 epoch 0 if n == 2, and no other use of the memory came in between.  Flags carry the
-                                 epoch and the ticket counters exist once per parity, so the kernel leaves what the next
-                                 epoch needs at zero by itself.  Only calls that ran the chain kernel count (see
-                                 used_workspace).  Start again from 0 before n would overflow. */
+                                 epoch 0 if n == 2, no other use of the memory came in between, and this call has no more
+                                 (state tile, chunk) pairs -- batch * nheads * headdim / 32 * nchunks -- than the epoch-0
+                                 call that cleared the workspace last (the flags behind those it cleared hold
+                                 anything).  Flags carry the epoch and the ticket counters exist once per parity, so the
+                                 kernel leaves what the next epoch needs at zero by itself.  Only calls that ran the chain
+                                 kernel count (see used_workspace).  Start again from 0 before n would overflow, and
+                                 whenever a call needs more pairs than the last clearing covered.  A broken promise is
+                                 detected by the kernel where it can be (wrong epoch before, flags outside the cleared
+                                 part) and reported as SSD_ERR_CHAIN_WORKSPACE by ssd_fused_workspace_status. */
     int32_t *used_workspace;  /* host memory or NULL: set to 1 if the call ran the chain kernel -- and so used the
                                  workspace and its epoch --, to 0 if another kernel family served it */
 } ssd_fused_opts;
@@ -190,13 +199,26 @@ int ssd_fused_chunk_state_passing_fwd_ws(const ssd_tensor *x, const ssd_tensor *
                                          const ssd_dims *dims, int clamp, const ssd_fused_opts *opts, void *stream);
 
 /*
- * Waits for `stream` and reads the error word of a workspace used by ssd_fused_chunk_state_passing_fwd_ws:
- * SSD_OK, or SSD_ERR_CHAIN_TIMEOUT when a wave of the last launch of the chain kernel on this workspace gave up
- * waiting (the outputs are then unusable).  A call that ran another kernel family (SSD_KERNEL_AUTO: see
- * ssd_query_fused_plan) leaves the workspace alone; memory the chain kernel has never cleared reports SSD_OK.
- * No counterpart in the reference, whose spin loops are unbounded (kernels/fused_concurrent.py:11, 300).
+ * Waits for `stream` and reads what the last launch of the chain kernel left in the header of a workspace used by
+ * ssd_fused_chunk_state_passing_fwd_ws: SSD_OK, or -- the outputs are then unusable --
+ *   SSD_ERR_CHAIN_WORKSPACE   the workspace was not what the call's epoch promised (another epoch before it, or more
+ *                             (state tile, chunk) pairs than the last clearing covered);
+ *   SSD_ERR_CHAIN_XCD         workgroups that report different XCDs drew from one per-XCD ticket counter (the LOCAL
+ *                             variant's assumption about the device does not hold);
+ *   SSD_ERR_CHAIN_INCOMPLETE  a ticket counter handed out fewer work items than it owns (LOCAL: an XCD that owns
+ *                             state tiles received no workgroup), so part of the outputs was never written;
+ *   SSD_ERR_CHAIN_TIMEOUT     a wave gave up waiting for the state entering its work item.
+ * Read it before the next launch on the same workspace, which starts the record afresh.  A call that ran another
+ * kernel family (SSD_KERNEL_AUTO: see ssd_query_fused_plan) leaves the workspace alone; memory the chain kernel has
+ * never cleared reports SSD_OK.  No counterpart in the reference, whose spin loops are unbounded and whose failure mode
+ * is a hang (kernels/fused_concurrent.py:11, 300).
+ * ssd_fused_workspace_status_of decodes a host copy of the first SSD_WORKSPACE_HEADER_INTS ints of a workspace the
+ * same way, for a caller that brings the header back with a copy of its own (no synchronisation here, no device
+ * needed).
  */
+#define SSD_WORKSPACE_HEADER_INTS 128
 int ssd_fused_workspace_status(const void *workspace, void *stream);
+int ssd_fused_workspace_status_of(const int32_t *header);
 
 /*
  * ssd_fused_chunk_state_passing_fwd_ws without a workspace argument and without any allocation.  It has no
@@ -330,6 +352,14 @@ int ssd_set_scan_kernel(int kernel);
  * another order), not bit for bit.
  */
 int ssd_set_token_split(int waves);
+
+/*
+ * Test hook with no counterpart in the reference: the number of XCDs (L2 caches) the LOCAL variant of the ticket /
+ * flag-chain kernel deals its units to; 0 = compute units / 32 (the default; 8 on MI355X), at most 16.  A wrong count
+ * is what the kernel's own checks exist for (SSD_ERR_CHAIN_XCD, SSD_ERR_CHAIN_INCOMPLETE) and how the tests provoke
+ * them.  Process-wide and atomic like the hooks below.  Returns the previous setting, or SSD_ERR_SHAPE.
+ */
+int ssd_set_chain_xcds(int xcds);
 
 /*
  * Tuning / test hook with no counterpart in the reference: how many consecutive chunks a workgroup of the

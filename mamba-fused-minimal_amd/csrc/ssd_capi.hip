@@ -363,6 +363,9 @@ const char *ssd_status_string(int status)
         case SSD_ERR_DEVICE: return "no gfx950 device is current";
         case SSD_ERR_SCRATCH: return "workspace missing or too small for the requested kernel";
         case SSD_ERR_CHAIN_TIMEOUT: return "a wave of the flag-chain kernel gave up waiting for its predecessor";
+        case SSD_ERR_CHAIN_XCD: return "workgroups of two XCDs drew from one ticket counter of the flag-chain kernel";
+        case SSD_ERR_CHAIN_INCOMPLETE: return "a ticket counter of the flag-chain kernel was never served: outputs are missing";
+        case SSD_ERR_CHAIN_WORKSPACE: return "the workspace was not in the state the epoch of the call promised";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -488,14 +491,21 @@ int ssd_fused_workspace_status(const void *workspace, void *stream)
     if (!workspace) return SSD_ERR_NULL;
     int rc = check_device();
     if (rc) return rc;
-    static_assert(ssd::kChainWsEpochWord == ssd::kChainWsErrWord + 2 && ssd::kChainWsTagWord == ssd::kChainWsErrWord + 3, "read in one copy");
-    int word[4] = {0, 0, 0, 0};       // error words of both parities, epoch of the last launch, tag
-    hipError_t e = hipMemcpyAsync(word, (const int *)workspace + ssd::kChainWsErrWord, sizeof(word), hipMemcpyDeviceToHost,
-                                  (hipStream_t)stream);
+    int32_t header[SSD_WORKSPACE_HEADER_INTS];
+    memset(header, 0, sizeof(header));
+    hipError_t e = hipMemcpyAsync(header, workspace, sizeof(header), hipMemcpyDeviceToHost, (hipStream_t)stream);
     if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return (int)e;
-    if (word[3] != ssd::kChainWsTag) return SSD_OK;      // the chain kernel has not run on this memory: nothing to report
-    return word[word[2] & 1] ? SSD_ERR_CHAIN_TIMEOUT : SSD_OK;
+    return ssd_fused_workspace_status_of(header);
+}
+
+int ssd_fused_workspace_status_of(const int32_t *header)
+{
+    static_assert(SSD_WORKSPACE_HEADER_INTS == ssd::kChainWsHeaderInts, "the header as the kernel lays it out");
+    static_assert(SSD_ERR_CHAIN_TIMEOUT == -7 && SSD_ERR_CHAIN_XCD == -8 && SSD_ERR_CHAIN_INCOMPLETE == -9 &&
+                  SSD_ERR_CHAIN_WORKSPACE == -10, "values chain_status_of_header returns");
+    if (!header) return SSD_ERR_NULL;
+    return ssd::chain_status_of_header(header);
 }
 
 int ssd_fused_cumsum_chunk_state_passing_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt_raw,
@@ -683,6 +693,12 @@ int ssd_set_scan_kernel(int kernel)
 {
     if (kernel < 0 || kernel > 2) return SSD_ERR_SHAPE;
     return ssd::set_scan_kernel(kernel);
+}
+
+int ssd_set_chain_xcds(int xcds)
+{
+    if (xcds < 0 || xcds > ssd::kChainMaxXcd) return SSD_ERR_SHAPE;
+    return ssd::set_chain_xcds(xcds);
 }
 
 int ssd_set_segment_chunks(int chunks)

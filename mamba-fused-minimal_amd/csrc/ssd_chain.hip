@@ -63,7 +63,7 @@ template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * N
 //    read-back loads and the flags carry the device-scope cache policy (sc1: written through to memory, read around
 //    the L2), nothing is flushed.  A link costs memory latencies (about 9 us measured).
 constexpr int kAuxDevice = 16;      // sc1
-constexpr int kMaxXcd = 16;
+constexpr int kMaxXcd = kChainMaxXcd;
 
 // workspace layout: ssd_params.h
 constexpr int kWsHeaderInts = kChainWsHeaderInts, kWsOwner = kChainWsOwnerWord;
@@ -135,11 +135,14 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     // chunk whose requests fetch nothing)
     auto decode = [&](int t, int r) {
         Item I;
-        const int tv = t < total ? t : 0;
+        // a ticket is an index into this slot's items; anything else (past the end, or a negative value that no
+        // counter hands out) gives the invalid chunk and never reaches the address arithmetic below
+        const bool in_range = (unsigned)t < (unsigned)total;
+        const int tv = in_range ? t : 0;
         const int k = tv / n_units;
         I.c = k * R + r;
         I.r = r;
-        I.valid = t < total && I.c < C;
+        I.valid = in_range && I.c < C;
         if (!I.valid) I.c = 0;
         I.tile = 4 * (unit0 + tv - k * n_units) + wave;
         const int r1 = I.tile / n_pt;
@@ -444,7 +447,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             while (load_flag(flag + c0) != epoch) {
                 __builtin_amdgcn_s_sleep(1);
                 if (++polls >= p.spin_limit) {
-                    if (lane == 0) __hip_atomic_fetch_or(ws_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (lane == 0) __hip_atomic_fetch_or(ws_err, kChainErrTimeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     break;
                 }
             }
@@ -499,17 +502,31 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     // a first item of a single chunk needs its successor from its first steps on and draws it here.
     if (threadIdx.x == 0) {
         const int t = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int c_first = (t < total ? t / n_units : 0) * R;
+        const int c_first = ((unsigned)t < (unsigned)total ? t / n_units : 0) * R;
         const bool single = !(R > 1 && c_first + 1 < C);
         tq[0] = t;
         tq[1] = single ? __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -1;
-        if (t == 0 && slot == 0) {
-            // one thread per launch: what the next launch on this workspace (epoch + 1, the other parity) must find
-            // at zero -- nothing of it is touched by this launch
+        if (t == 0) {
+            // One thread per slot and launch (all of them write the same values, so that the launch does not depend
+            // on a particular slot being served).  First: is the workspace what the epoch promises?  The launch
+            // before must have been epoch - 1 (a clearing leaves 0), and the flags this launch looks at must lie
+            // inside what the last clearing covered -- beyond it the memory holds anything, possibly this epoch.
+            const int before = __hip_atomic_load(p.ws + kChainWsEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int cleared = __hip_atomic_load(p.ws + kChainWsClearedWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((before != epoch - 1 && before != epoch) || (int64_t)cleared < kWsHeaderInts + (int64_t)p.n_items * p.C)
+                __hip_atomic_fetch_or(ws_err, kChainErrWorkspace, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // What the next launch on this workspace (epoch + 1, the other parity) must find at zero -- nothing of
+            // it is touched by this launch --, and how many items each slot of this launch has to hand out.
             int *const other = p.ws + kChainWsBankStride * (bank ^ 1);
-            for (int i = 0; i < kMaxXcd; ++i) __hip_atomic_store(other + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < kChainWsBankStride; ++i) __hip_atomic_store(other + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.ws + kChainWsErrWord + (bank ^ 1), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.ws + kChainWsEpochWord, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int *const totals = p.ws + kChainWsBankStride * bank + kChainWsTotalOffset;
+            const int all_units = p.n_items >> 2, slots = LOCAL ? p.n_xcd : 1;
+            for (int i = 0; i < kMaxXcd; ++i) {
+                const int u = i < slots ? all_units / slots + (i < all_units % slots ? 1 : 0) : 0;
+                __hip_atomic_store(totals + i, u * n_super, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
     // rows past the end of the sequence are not fetched and leave their LDS slots untouched; their weight is zero,
@@ -527,7 +544,16 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     if (second_late) t_nxt = total;              // no item; not looked at before the ticket is there
     Item cur = decode(t_cur, 0);
     Item nxt = successor(cur, t_cur, t_nxt);
-    if (!cur.valid) return;                      // whole workgroup: no barrier is skipped
+    if (!cur.valid) {                            // whole workgroup: no barrier is skipped
+        // Nothing to do -- or ticket counters that an earlier launch of the same parity left behind (an epoch that does
+        // not follow the one before): then nobody draws ticket 0, and this is where the broken promise shows.
+        if (threadIdx.x == 0) {
+            const int before = __hip_atomic_load(p.ws + kChainWsEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before != epoch - 1 && before != epoch)
+                __hip_atomic_fetch_or(ws_err, kChainErrWorkspace, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
 
     Meta mcur = load_meta(cur);
     // requests of the steps 0..kDist-1, in the order (x, x, B...) that every later step keeps
@@ -668,7 +694,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         // every workgroup that drew from a slot's counter must sit on the same XCD; anything else (hardware ids that
         // do not spread over p.n_xcd slots) would break the L2 argument above, and is reported instead of ignored
         const int seen = __hip_atomic_fetch_max(p.ws + kWsOwner + slot, xcd_hw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (seen != 0 && seen != xcd_hw + 1) __hip_atomic_fetch_or(ws_err, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (seen != 0 && seen != xcd_hw + 1) __hip_atomic_fetch_or(ws_err, kChainErrXcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -676,7 +702,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 // this kernel's (a workspace may hold anything before its first launch)
 __global__ void __launch_bounds__(256) clear_kernel(int *ws, int n)
 {
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = chain_workspace_clear(i);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) ws[i] = chain_workspace_clear(i, n);
 }
 
 static bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
@@ -686,7 +712,33 @@ static bool rows_ok(const void *ptr, int64_t strides_or, int64_t row_stride, int
     return aligned(ptr, 16) && strides_or % 4 == 0 && (int64_t)headdim * row_stride < (1LL << 28);
 }
 
+// LOCAL reads passed states back with plain loads, which the per-CU cache may serve: safe as long as a compute unit
+// never holds a line that another wave's tile shares, i.e. as long as every row that is read back (of fp32 `out`, or
+// of the fp32 slots of the workspace when `out` is 16-bit) starts and ends on 128-byte line boundaries.
+static bool local_lines_ok(const Params &p)
+{
+    if (p.dt_out != DT_F32) return aligned(p.ws, 128);        // slots: 256-byte offset, 32 x dstate x 4 bytes each
+    const int64_t strides_or = p.so_b | p.so_c | p.so_h | p.so_p | p.dstate;
+    return aligned(p.out, 128) && (strides_or * 4) % 128 == 0;
+}
+
+static std::atomic<int> g_forced_xcds{0};
+
 }  // namespace chain
+
+int set_chain_xcds(int n) { return chain::g_forced_xcds.exchange(n); }
+
+// bit 2 first: with a workspace that is not what the epoch promised, the other words mean nothing
+int chain_status_of_header(const int *h)
+{
+    if (h[kChainWsTagWord] != kChainWsTag) return 0;       // the chain kernel has not run on this memory
+    const int bank = h[kChainWsEpochWord] & 1, err = h[kChainWsErrWord + bank];
+    if (err & kChainErrWorkspace) return -10;
+    if (err & kChainErrXcd) return -8;
+    for (int s = 0; s < kChainMaxXcd; ++s)
+        if (h[kChainWsBankStride * bank + s] < h[kChainWsBankStride * bank + kChainWsTotalOffset + s]) return -9;
+    return (err & kChainErrTimeout) ? -7 : 0;
+}
 
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks)
 {
@@ -794,6 +846,8 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     // the fullest XCD holds at most an eighth more than its fair share of them.
     const int n_units = p.n_items >> 2;
     p.n_xcd = n_cu >= 32 ? n_cu / 32 : 1;
+    const int forced_xcds = chain::g_forced_xcds.load(std::memory_order_relaxed);
+    if (forced_xcds > 0) p.n_xcd = forced_xcds;      // test hook: a wrong count is what the kernel's checks are for
     if (p.n_xcd > chain::kMaxXcd) p.n_xcd = chain::kMaxXcd;
     // LOCAL when the units spread evenly over the XCDs and each has a few of its own: producer and consumer of a passed
     // state then share an L2 (no read-back from memory), and an XCD only fetches the B rows of its own units' groups
@@ -801,7 +855,7 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     // against 1.17 ms).  With one or
     // two units per XCD most of its workgroups would sit in one chain.
     const int fullest = (n_units + p.n_xcd - 1) / p.n_xcd;
-    const bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
+    bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
     // Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units
     // end up with too few or too unequal numbers of items that large.  p.n_seg > 0 forces a value.
     const int r = chain_chunks_per_item(p, n_cu, p.n_seg);
@@ -809,6 +863,8 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
         if (r < 2) return hipErrorInvalidValue;
         p.carry = (float *)(p.ws + carry_offset_ints(p.n_items, p.C));
     }
+    // buffers whose tiles share cache lines (an `out` view at an odd offset): through memory, also where LOCAL was asked for
+    if (local && !chain::local_lines_ok(p)) local = false;
     const int64_t total = (int64_t)n_units * ((p.C + r - 1) / r);
     int n_wg = (int)(total < n_cu ? total : n_cu);
     // LOCAL: a workgroup only works on the units of the XCD it finds itself on, so every XCD needs one.  Workgroups go

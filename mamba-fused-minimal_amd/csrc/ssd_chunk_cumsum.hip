@@ -33,7 +33,7 @@ __global__ void __launch_bounds__(256) chunk_cumsum_kernel(const CumsumParams p)
     if (p.clear) {
         // on the way: the workspace of the chain kernel that this launch is in front of
         const int n_wg = gridDim.x * gridDim.y * gridDim.z, wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-        for (int i = wg * 256 + tid; i < p.n_clear; i += n_wg * 256) p.clear[i] = chain_workspace_clear(i);
+        for (int i = wg * 256 + tid; i < p.n_clear; i += n_wg * 256) p.clear[i] = chain_workspace_clear(i, p.n_clear);
     }
 
     auto activate = [&](float d) {

@@ -175,22 +175,36 @@ int chain_chunks_per_item(const Params &p, int n_cu, int forced);     // what la
 
 // Layout of a chain workspace (ints).  A launch carries an epoch, one more than that of the launch before it on the
 // same workspace.  Everything a launch must find in a known state is either tagged with the epoch or kept twice:
-//   [32 b + slot]  ticket counters, one bank b = epoch & 1 per parity, a slot per XCD (16).  The workgroup that draws
-//                  ticket 0 of slot 0 zeroes the other bank, the other error word and records the epoch: the next
+//   [32 b + slot]  ticket counters, one bank b = epoch & 1 per parity, a slot per XCD (16).  The workgroups that draw
+//                  ticket 0 of a slot zero the other bank, the other error word and record the epoch: the next
 //                  launch finds its counters at zero without a fill launch in between.
-//   [64 + b]       error word of the launch with parity b;  [66] epoch of the last launch;  [67] a tag that says a
-//                  chain launch has cleared this memory at least once (without it the words above mean nothing)
+//   [32 b + 16 + slot]  work items each slot has to hand out in the launch with parity b (written with the above): a
+//                  slot whose counter ends below it was never served (ssd_fused_workspace_status)
+//   [64 + b]       error word of the launch with parity b (bit 0: a flag wait ran out, bit 1: two XCDs drew from one
+//                  slot, bit 2: the workspace is not in the state the epoch promises);  [66] epoch of the last launch;
+//                  [67] a tag that says a chain launch has cleared this memory at least once (without it the words
+//                  above mean nothing);  [68] ints cleared by the last clearing (flags beyond hold anything)
 //   [96 + slot]    hardware id (+1) of the XCD that drew from each slot
 //   [128 ...]      flags, one per (state tile, chunk): raised = holds the epoch of the launch (older values, from
 //                  launches before, and the zeros of a clearing never equal it)
 //   behind the flags, from the next multiple of 64 ints: 32 x dstate fp32 per (state tile, item) when `out` is bf16;
 //                  written before it is read in every launch, never cleared
-constexpr int kChainWsHeaderInts = 128, kChainWsBankStride = 32, kChainWsErrWord = 64, kChainWsEpochWord = 66,
-              kChainWsTagWord = 67, kChainWsOwnerWord = 96, kChainWsTag = 0x53534443;
-// The value a cleared chain workspace holds at int i: zero, except for the tag.  Any kernel that runs in front of the
-// chain kernel on the same stream may do the clearing (the stand-alone producer of dt / dA_cumsum does when both are
-// launched by one call); Params::ws_cleared then keeps the chain kernel's own fill launch away.
-__host__ __device__ constexpr int chain_workspace_clear(int i) { return i == kChainWsTagWord ? kChainWsTag : 0; }
+constexpr int kChainWsHeaderInts = 128, kChainWsBankStride = 32, kChainWsTotalOffset = 16, kChainWsErrWord = 64,
+              kChainWsEpochWord = 66, kChainWsTagWord = 67, kChainWsClearedWord = 68, kChainWsOwnerWord = 96,
+              kChainWsTag = 0x53534443, kChainMaxXcd = 16;
+enum : int { kChainErrTimeout = 1, kChainErrXcd = 2, kChainErrWorkspace = 4 };
+// The value a clearing of the first n ints of a chain workspace leaves at int i: zero, except for the tag and the
+// record of n itself.  Any kernel that runs in front of the chain kernel on the same stream may do the clearing (the
+// stand-alone producer of dt / dA_cumsum does when both are launched by one call); Params::ws_cleared then keeps the
+// chain kernel's own fill launch away.
+__host__ __device__ constexpr int chain_workspace_clear(int i, int n)
+{
+    return i == kChainWsTagWord ? kChainWsTag : i == kChainWsClearedWord ? n : 0;
+}
+// What the first kChainWsHeaderInts ints of a workspace say about the last chain launch on it: 0, or the most
+// serious of the conditions above as a negative ssd_status.  Host logic.
+int chain_status_of_header(const int *header);
+int set_chain_xcds(int n);        // 0 = from the device's compute units; a test hook; returns the old value
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

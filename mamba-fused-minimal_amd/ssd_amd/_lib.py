@@ -14,7 +14,7 @@ _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
            "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes", "ssd_fused_workspace_bytes_for",
-           "ssd_fused_workspace_status", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
+           "ssd_fused_workspace_status", "ssd_fused_workspace_status_of", "ssd_set_chain_xcds", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
            "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd_ws", "ssd_query_path", "ssd_query_fused_plan", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
@@ -39,7 +39,8 @@ class SsdFusedPlan(ctypes.Structure):
 
 SSD_FAMILIES = ("generic", "token_split", "four_tile", "pair", "chain")
 SSD_KERNEL_AUTO, SSD_KERNEL_CHAIN, SSD_KERNEL_CHAIN_LOCAL, SSD_KERNEL_CHAIN_GLOBAL = 0, 1, 2, 3
-SSD_ERR_SCRATCH, SSD_ERR_CHAIN_TIMEOUT = -6, -7
+SSD_ERR_SCRATCH, SSD_ERR_CHAIN_TIMEOUT, SSD_ERR_CHAIN_XCD, SSD_ERR_CHAIN_INCOMPLETE, SSD_ERR_CHAIN_WORKSPACE = -6, -7, -8, -9, -10
+SSD_WORKSPACE_HEADER_INTS = 128
 
 _lib = None
 
@@ -72,6 +73,10 @@ def load():
     lib.ssd_fused_workspace_bytes_for.argtypes = [D, ctypes.c_int, ctypes.c_int]
     lib.ssd_fused_workspace_status.restype = ctypes.c_int
     lib.ssd_fused_workspace_status.argtypes = [vp, vp]
+    lib.ssd_fused_workspace_status_of.restype = ctypes.c_int
+    lib.ssd_fused_workspace_status_of.argtypes = [ctypes.POINTER(ctypes.c_int32)]
+    lib.ssd_set_chain_xcds.restype = ctypes.c_int
+    lib.ssd_set_chain_xcds.argtypes = [ctypes.c_int]
     lib.ssd_fused_chunk_state_passing_fwd_static.restype = ctypes.c_int
     lib.ssd_fused_chunk_state_passing_fwd_static.argtypes = [T, T, T, T, T, T, T, T, D, ctypes.c_int, vp]
     lib.ssd_fused_static_status.restype = ctypes.c_int

@@ -23,44 +23,64 @@ def _stream(t):
 # Workspaces of the ticket / flag-chain kernel that the wrappers keep to themselves: one per (device, stream), grown on
 # demand, with the epoch of the last launch on it.  A workspace nobody else writes to lets a call tell the library that
 # the launch before left it in order (ssd_fused_opts.epoch), which saves the fill launch in front of the kernel.
-_WORKSPACES = {}
-_WORKSPACES_LOCK = threading.Lock()
+_WORKSPACES = {}                       # (device index, stream handle) -> _Kept
+_WORKSPACES_LOCK = threading.Lock()    # guards the dictionary only; a launch holds its entry's own lock
 
 
 class _Epochs:
     """The epochs of one kept workspace as ssd_fused_opts.epoch wants them: 0 for the first call (the library clears the
     workspace and counts the call as epoch 1), then 2, 3, ... -- but only calls that ran the chain kernel count, a failed
-    call makes the contents unknown again, and the count starts over before it could overflow."""
+    call makes the contents unknown again, the count starts over before it could overflow, and a call that looks at
+    more flags than the last clearing covered (more state tiles x chunks than the call that was given epoch 0) clears
+    again: the flags beyond hold whatever the memory held before, possibly the value of the coming epoch."""
     LIMIT = 1 << 30
 
     def __init__(self):
         self.last = 0                      # epoch of the last chain launch on the workspace; 0 = contents unknown
+        self.cleared = 0                   # (state tile, chunk) pairs whose flags the last clearing covered
 
-    def next(self):
-        if self.last >= self.LIMIT:
+    def next(self, pairs):
+        if self.last >= self.LIMIT or pairs > self.cleared:
             self.last = 0
         return 0 if self.last == 0 else self.last + 1
 
-    def done(self, epoch, rc, used_workspace):
+    def done(self, epoch, rc, used_workspace, pairs):
         if rc:
             self.last = 0
+            self.cleared = 0
         elif used_workspace:
             self.last = max(epoch, 1)
+            if epoch <= 0:
+                self.cleared = pairs
+
+
+class _Kept:
+    """A workspace the wrappers keep for one (device, stream), the epochs of the launches on it and the lock that
+    keeps those launches in order (epochs must reach the stream in the order they were handed out)."""
+
+    def __init__(self, tensor):
+        self.tensor = tensor
+        self.epochs = _Epochs()
+        self.lock = threading.Lock()
+
+
+def _workspace_key(device, stream=None):
+    stream = torch.cuda.current_stream(device) if stream is None else stream
+    return (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
 
 
 def _own_workspace(x, nbytes):
-    """-> (int32 tensor, its _Epochs or None).  Call with _WORKSPACES_LOCK held, and keep it until the launch is
-    enqueued: the epochs must reach the stream in order."""
-    stream = torch.cuda.current_stream(x.device)
+    """-> the _Kept of x's device and current stream, holding at least nbytes (None under stream capture)."""
     if torch.cuda.is_current_stream_capturing():
         # a captured launch is replayed with the same arguments: the same epoch again and again would take the flags of
         # the replay before for its own.  Epoch 0 (clear every time) is what a graph needs.
-        return torch.empty(((nbytes + 3) // 4,), device=x.device, dtype=torch.int32), None
-    key = (x.device.index, stream.cuda_stream)
-    ent = _WORKSPACES.get(key)
-    if ent is None or ent[0].numel() * 4 < nbytes:
-        ent = (torch.empty((max(nbytes, 1 << 16) + 3) // 4, device=x.device, dtype=torch.int32), _Epochs())
-        _WORKSPACES[key] = ent
+        return None
+    key = _workspace_key(x.device)
+    with _WORKSPACES_LOCK:
+        ent = _WORKSPACES.get(key)
+        if ent is None or ent.tensor.numel() * 4 < nbytes:
+            ent = _Kept(torch.empty((max(nbytes, 1 << 16) + 3) // 4, device=x.device, dtype=torch.int32))
+            _WORKSPACES[key] = ent
     return ent
 
 
@@ -72,16 +92,37 @@ def release_workspaces():
         _WORKSPACES.clear()
 
 
-def _launch_on_own_workspace(x, nbytes, launch, used):
-    """Runs launch(workspace, epoch) -> status on the wrappers' workspace for x's device and stream."""
-    with _WORKSPACES_LOCK:
-        workspace, epochs = _own_workspace(x, nbytes)
-        if epochs is None:
-            return launch(workspace, 0)
-        epoch = epochs.next()
-        rc = launch(workspace, epoch)
-        epochs.done(epoch, rc, used.value)
+def _launch_on_own_workspace(x, nbytes, launch, used, pairs):
+    """Runs launch(workspace, epoch) -> status on the wrappers' workspace for x's device and stream.  pairs: the
+    (state tile, chunk) pairs of the call, i.e. the flags it looks at.  Only launches on the same device and stream
+    wait for each other here."""
+    ent = _own_workspace(x, nbytes)
+    if ent is None:
+        return launch(torch.empty(((nbytes + 3) // 4,), device=x.device, dtype=torch.int32), 0)
+    with ent.lock:
+        epoch = ent.epochs.next(pairs)
+        rc = launch(ent.tensor, epoch)
+        ent.epochs.done(epoch, rc, used.value, pairs)
         return rc
+
+
+def fused_status(device=None, stream=None):
+    """What the last fused call of this module on ``device`` and ``stream`` (defaults: the current ones) left in the
+    workspace the wrappers keep for them: waits for the stream and returns 0, or the negative ssd_status of
+    ssd_fused_workspace_status (-7 a flag wait ran out, -8 two XCDs drew from one counter, -9 a counter that owns work
+    was never served, -10 the workspace was not what the epoch promised) -- the outputs of that call are then
+    unusable.  Ask before the next fused call on the same stream, which starts the record afresh.  0 also when no call
+    has used that workspace (another kernel family served it).  The reference's fused kernels have no such report:
+    their spin loops are unbounded and a failure is a hang (kernels/fused_concurrent.py:11, 300)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    stream = torch.cuda.current_stream(device) if stream is None else stream
+    with _WORKSPACES_LOCK:
+        ent = _WORKSPACES.get(_workspace_key(device, stream))
+    if ent is None:
+        return 0
+    with ent.lock, torch.cuda.device(device):
+        return int(_lib.load().ssd_fused_workspace_status(ctypes.c_void_p(ent.tensor.data_ptr()),
+                                                          ctypes.c_void_p(stream.cuda_stream)))
 
 
 def _prep_inputs(B, x, dt, dA_cumsum, seq_idx):
@@ -232,7 +273,8 @@ def _fused_chunk_state_state_passing_fwd(B, x, dt, dA_cumsum, out_dtype, initial
         nbytes = 0
         if states is None:          # with a `states` buffer the call runs on other kernels anyway
             nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out_dtype, -1), int(_chunks_per_item)))
-        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
+        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used,
+                                      batch * nheads * ((headdim + 31) // 32) * nchunks)
     _lib.check(rc, "ssd_fused_chunk_state_passing_fwd_ws")
     return out, final_states
 
@@ -276,8 +318,8 @@ def _fused_static_status(device=None):
 
 
 def _fused_workspace_status(workspace):
-    """Waits for the current stream and returns 0, or -7 if a flag wait of the last fused launch that used
-    ``workspace`` ran out (ssd_fused_workspace_status)."""
+    """Waits for the current stream and returns 0, or the negative status of the last fused launch that used
+    ``workspace`` (ssd_fused_workspace_status: -7 ... -10)."""
     with torch.cuda.device(workspace.device):
         return int(_lib.load().ssd_fused_workspace_status(ctypes.c_void_p(workspace.data_ptr()), _stream(workspace)))
 
@@ -387,7 +429,8 @@ def _fused_cumsum_chunk_state_state_passing_fwd(B, x, dt, A, chunk_size, out_dty
         rc = launch(_workspace, 0)
     else:
         nbytes = int(lib.ssd_fused_workspace_bytes_for(dims, _lib._DTYPES.get(out.dtype, -1), int(_chunks_per_item)))
-        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used)
+        rc = _launch_on_own_workspace(x, nbytes or int(lib.ssd_fused_workspace_bytes(dims)), launch, used,
+                                      batch * nheads * ((headdim + 31) // 32) * nchunks)
     _lib.check(rc, "ssd_fused_cumsum_chunk_state_passing_fwd_ws")
     return out, final_states, dA_cumsum, dt_out
 
@@ -439,6 +482,16 @@ def set_scan_kernel(kernel):
     rc = _lib.load().ssd_set_scan_kernel(int(kernel))
     if rc < 0:
         raise ValueError("scan kernel must be 0, 1 or 2")
+    return rc
+
+
+def set_chain_xcds(xcds):
+    """Test hook (no counterpart in the reference): the number of XCDs the per-XCD variant of the ticket / flag-chain
+    kernel deals its units to; 0 = from the device.  A wrong count provokes the kernel's own checks
+    (fused_status -8 / -9).  Returns the previous setting."""
+    rc = _lib.load().ssd_set_chain_xcds(int(xcds))
+    if rc < 0:
+        raise ValueError("the number of XCDs must be 0 (from the device) .. 16")
     return rc
 
 

@@ -244,7 +244,7 @@ def test_kept_workspaces_can_be_released():
     import ssd_amd
     from ssd_amd import ops
     with ops._WORKSPACES_LOCK:
-        ops._WORKSPACES[("test", 0)] = (torch.zeros(4, dtype=torch.int32), ops._Epochs())
+        ops._WORKSPACES[("test", 0)] = ops._Kept(torch.zeros(4, dtype=torch.int32))
     ssd_amd.release_workspaces()
     assert not ops._WORKSPACES
 
@@ -253,19 +253,76 @@ def test_epochs_of_a_kept_workspace():
     # what the wrappers pass as ssd_fused_opts.epoch for the workspace they keep per device and stream
     from ssd_amd.ops import _Epochs
     e = _Epochs()
-    assert e.next() == 0                                   # contents unknown: the library clears, the call counts as 1
-    e.done(0, 0, 1)
-    assert e.next() == 2
-    e.done(2, 0, 1)
-    assert e.next() == 3
-    e.done(3, 0, 0)                                        # another kernel family served the call: the epoch was not used
-    assert e.next() == 3
-    e.done(3, 0, 1)
-    assert e.next() == 4
-    e.done(4, -6, 0)                                       # a failed call: contents unknown again
-    assert e.next() == 0
-    e.done(0, 0, 0)                                        # cleared by nobody (not the chain kernel): still unknown
-    assert e.next() == 0
-    e.done(0, 0, 1)
+    assert e.next(100) == 0                                # contents unknown: the library clears, the call counts as 1
+    e.done(0, 0, 1, 100)
+    assert e.next(100) == 2
+    e.done(2, 0, 1, 100)
+    assert e.next(50) == 3                                 # fewer flags than the clearing covered: fine
+    e.done(3, 0, 0, 50)                                    # another kernel family served the call: the epoch was not used
+    assert e.next(100) == 3
+    e.done(3, 0, 1, 100)
+    assert e.next(100) == 4
+    e.done(4, -6, 0, 100)                                  # a failed call: contents unknown again
+    assert e.next(100) == 0
+    e.done(0, 0, 0, 100)                                   # cleared by nobody (not the chain kernel): still unknown
+    assert e.next(100) == 0
+    e.done(0, 0, 1, 100)
     e.last = _Epochs.LIMIT                                 # before the count could overflow it starts over
-    assert e.next() == 0
+    assert e.next(100) == 0
+    e.done(0, 0, 1, 100)
+    # a call that looks at more flags than the last clearing covered must not trust the ones beyond: clear again
+    assert e.next(100) == 2
+    e.done(2, 0, 1, 100)
+    assert e.next(101) == 0
+    e.done(0, 0, 1, 101)
+    assert e.next(101) == 2 and e.cleared == 101
+
+
+def _header(epoch, err=0, tickets=(), totals=(), tag=True):
+    """The first 128 ints of a chain workspace after a launch with this epoch (layout: csrc/ssd_params.h)."""
+    import ctypes
+    h = (ctypes.c_int32 * 128)()
+    bank = epoch & 1
+    for s, t in enumerate(tickets):
+        h[32 * bank + s] = t
+    for s, t in enumerate(totals):
+        h[32 * bank + 16 + s] = t
+    h[64 + bank] = err
+    h[66] = epoch
+    h[67] = 0x53534443 if tag else 0
+    return h
+
+
+def test_workspace_status_decoding():
+    """ssd_fused_workspace_status_of on host copies of a workspace header: every failure of the ticket / flag-chain
+    kernel has its own code, and a ticket counter that owns work items but handed out fewer (an XCD that received no
+    workgroup) is an error although no error bit is set."""
+    from ssd_amd import _lib
+    lib = _lib.load()
+    st = lib.ssd_fused_workspace_status_of
+    assert st(None) == -1
+    assert st(_header(3, tag=False, err=7)) == 0                                  # never a chain workspace
+    ok = dict(tickets=[40 + 32] * 8, totals=[40] * 8)                             # every workgroup draws one past the end
+    assert st(_header(3, **ok)) == 0
+    assert st(_header(4, **ok)) == 0                                              # the other parity
+    assert st(_header(3, err=1, **ok)) == _lib.SSD_ERR_CHAIN_TIMEOUT == -7
+    assert st(_header(3, err=2, **ok)) == _lib.SSD_ERR_CHAIN_XCD == -8
+    assert st(_header(3, err=3, **ok)) == -8
+    assert st(_header(3, err=4 | 1, **ok)) == _lib.SSD_ERR_CHAIN_WORKSPACE == -10
+    # slot 5 owns 40 items and handed out none / some
+    for drawn in (0, 39):
+        t = [72] * 8
+        t[5] = drawn
+        assert st(_header(3, tickets=t, totals=[40] * 8)) == _lib.SSD_ERR_CHAIN_INCOMPLETE == -9
+        assert st(_header(2, tickets=t, totals=[40] * 8)) == -9
+    t = [72] * 8
+    t[5] = 40
+    assert st(_header(3, tickets=t, totals=[40] * 8)) == 0
+    # slots without units need no workgroup (GLOBAL: one counter)
+    assert st(_header(3, tickets=[1536], totals=[1280])) == 0
+    # the error word of the other parity belongs to another launch
+    h = _header(3, **ok)
+    h[64] = 1
+    assert st(h) == 0
+    for code in (-7, -8, -9, -10):
+        assert lib.ssd_status_string(code).decode() not in ("unknown status", "")

@@ -26,12 +26,20 @@ class Workspace:
     two banks of ticket counters and two error words, by parity of the epoch; the epoch of the last launch; flags that
     hold the epoch they were raised in.  Cleared = all zero."""
 
-    def __init__(self, n_flags=4096):
+    def __init__(self, n_flags=4096, cleared=None, garbage=0):
         self.tickets = [0, 0]
         self.errors = [0, 0]
         self.last_epoch = 0
-        self.flags = [0] * n_flags
+        # a clearing covers the flags the call that asked for it looks at; what lies behind holds whatever the memory
+        # held before (`garbage`)
+        self.cleared = n_flags if cleared is None else cleared
+        self.flags = [0] * self.cleared + [garbage] * (n_flags - self.cleared)
         self.carry = [float("nan")] * n_flags      # exact copies of the states that cross between items; never cleared
+
+    def clear(self, n):
+        """What a call with epoch 0 does first: zero for the n flags it looks at, and a record of n."""
+        self.tickets, self.errors, self.last_epoch, self.cleared = [0, 0], [0, 0], 0, n
+        self.flags[:n] = [0] * n
 
     def status(self):
         return self.errors[self.last_epoch & 1]
@@ -90,6 +98,10 @@ class Launch:
         t = self.ws.tickets[self.bank]
         self.ws.tickets[self.bank] += 1
         if t == 0:
+            # is the workspace what the epoch promises?  The launch before was epoch - 1 (0 after a clearing), and the
+            # flags this launch looks at were covered by the last clearing
+            if self.ws.last_epoch != self.epoch - 1 or self.ws.cleared < self.n_units * (self.C + 1):
+                self.error |= 4
             # one workgroup per launch: what the next epoch (the other parity) must find at zero
             self.ws.tickets[self.bank ^ 1] = 0
             self.ws.errors[self.bank ^ 1] = 0
@@ -104,6 +116,10 @@ class Launch:
         """One persistent workgroup as a generator: every `yield` is a point where the scheduler may switch."""
         cur = self.draw()
         if cur >= self.total:
+            # nothing to do -- or counters that a launch two epochs back left behind, in which case nobody draws
+            # ticket 0 and this is where the broken promise shows
+            if self.ws.last_epoch not in (self.epoch - 1, self.epoch):
+                self.error |= 4
             return
         u, c0, c1 = self.item(cur)
         single = c1 - c0 == 1
@@ -283,3 +299,35 @@ def test_rounded_passed_states_cross_between_items_exactly():
             for c in range(C):
                 assert abs(L.out[u][c] - L.rnd(want[u][c])) <= (1e-2 + 1e-9 if L.rounded else 1e-12 * max(1.0, abs(want[u][c]))), (i, u, c)
         epoch += 1
+
+
+def test_flags_behind_the_cleared_part_are_not_trusted():
+    """A kept workspace is cleared for the call that starts its epochs; a later call with more (unit, chunk) pairs looks
+    at flags behind that part, which hold whatever the memory held -- here the very value of the coming epoch, so
+    every wait would be skipped.  The kernel's check at ticket 0 reports it; the host policy of the wrappers (clear again
+    when a call needs more flags than the last clearing covered) avoids it."""
+    small, big = (3, 5, 1, 8), (7, 9, 2, 16)
+    n_small, n_big = small[0] * (small[1] + 1), big[0] * (big[1] + 1)
+    wrong = 0
+    for seed in range(10):
+        ws = Workspace(cleared=n_small, garbage=2)
+        Launch(*small, 1000, spin_limit=1 << 30, seed=seed, ws=ws, epoch=1).run()
+        assert ws.status() == 0
+        L = Launch(*big, 1000, spin_limit=1 << 30, seed=50 + seed, ws=ws, epoch=2).run()
+        assert ws.status() & 4                       # reported ...
+        want = L.reference()
+        wrong += any(L.out[u][c] is None or not abs(L.out[u][c] - want[u][c]) <= 1e-9 for u in range(big[0]) for c in range(big[1] + 1))
+        # the host policy: this call needs more flags than were cleared -> epoch 0, i.e. clear, then launch as epoch 1
+        ws = Workspace(cleared=n_small, garbage=2)
+        Launch(*small, 1000, spin_limit=1 << 30, seed=seed, ws=ws, epoch=1).run()
+        ws.clear(n_big)
+        L = Launch(*big, 2, spin_limit=1 << 30, seed=50 + seed, ws=ws, epoch=1).run()
+        assert ws.status() == 0
+        want = L.reference()
+        assert all(abs(L.out[u][c] - want[u][c]) <= 1e-12 * max(1.0, abs(want[u][c])) for u in range(big[0]) for c in range(big[1] + 1))
+    assert wrong > 0                                 # ... and with reason: skipped waits do give wrong states
+    # an epoch that does not follow the one before is reported as well
+    ws = Workspace()
+    Launch(*small, 1000, spin_limit=1 << 30, seed=0, ws=ws, epoch=1).run()
+    Launch(*small, 1000, spin_limit=1 << 30, seed=1, ws=ws, epoch=3).run()
+    assert ws.status() & 4

@@ -340,12 +340,17 @@ def test_chain_workspace_kept_across_calls_with_epochs(ops, oracle):
              (dict(L=2304, H=8), LOCAL, 1), (dict(b=1, L=4096, H=16), GLOBAL, 4), (dict(b=2, L=2048, H=8, init=True), LOCAL, 2),
              (dict(P=128, H=4, G=2, L=1280), LOCAL, 4), (dict(b=1, L=4096, H=16), LOCAL, 4), (dict(L=2304, H=8), GLOBAL, 4)]
     ws = torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda")
-    epoch = 0
+    epoch, cleared = 0, 0
     for i, (kw, kernel, r) in enumerate(cases * 2):
         d = oracle.make_inputs(3 if "nseq" in kw else 2, **kw)
         want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"],
                                               seq_idx=d["seq_idx"])
-        print(f"[epochs {i}] {kw} kernel={kernel} chunks/item={r} epoch={epoch}", flush=True)
+        # the promise of an epoch covers the flags the last clearing covered: a call with more (state tile, chunk) pairs
+        # starts over with epoch 0 (twice in this sequence)
+        pairs = d["x"].shape[0] * d["x"].shape[2] * (d["x"].shape[3] // 32) * d["dt"].shape[2]
+        if pairs > cleared:
+            epoch, cleared = 0, pairs
+        print(f"[epochs {i}] {kw} kernel={kernel} chunks/item={r} epoch={epoch} pairs={pairs}", flush=True)
         out, fin = ops._fused_chunk_state_state_passing_fwd(
             *[_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")], torch.float32, initial_states=_dev(d["initial_states"]),
             seq_idx=_dev(d["seq_idx"]), _kernel=kernel, _chunks_per_item=r, _workspace=ws, _epoch=epoch)
@@ -392,3 +397,116 @@ def test_wrapper_keeps_its_own_workspace(ops, oracle):
     st.synchronize()
     key = str(dict(b=1, L=8192, H=80))
     assert _mismatches(out, wants[key][0])[0] == 0 and _mismatches(fin, wants[key][1])[0] == 0
+
+
+def test_chain_reports_a_workspace_that_is_not_what_the_epoch_promises(ops, oracle):
+    """ssd_fused_opts.epoch > 0 promises that the launch before was epoch - 1 and that the call looks at no more flags
+    than the last clearing covered.  A small call clears 256 flags; a larger one with epoch 2 looks at 512, and the
+    memory behind the cleared part holds the value 2 -- every wait would be skipped.  The kernel notices at ticket 0 and
+    ssd_fused_workspace_status says so (SSD_ERR_CHAIN_WORKSPACE); an epoch that does not follow the one before is
+    reported too.  The wrappers' own workspace is not exposed to this: they clear again when a call needs more."""
+    from ssd_amd import ops as ops_module
+    small = oracle.make_inputs(2, b=2, L=2048, H=8)            # 32 state tiles x 8 chunks
+    big = oracle.make_inputs(2, b=1, L=4096, H=16)             # 32 x 16
+    want = oracle.fused_ref(big["B"], big["x"], big["dt"], big["dA_cumsum"], initial_states=big["initial_states"])
+    run = lambda d, **kw: ops._fused_chunk_state_state_passing_fwd(
+        *[_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")], torch.float32, initial_states=_dev(d["initial_states"]), **kw)
+    ws = torch.full((1 << 16,), 2, dtype=torch.int32, device="cuda")
+    run(small, _kernel=GLOBAL, _workspace=ws, _epoch=0)
+    assert ops._fused_workspace_status(ws) == 0
+    print("[promise] more flags than were cleared, epoch 2", flush=True)
+    run(big, _kernel=GLOBAL, _workspace=ws, _epoch=2, _spin_limit=64)
+    assert ops._fused_workspace_status(ws) == -10
+    # started over, the same call is clean
+    out, fin = run(big, _kernel=GLOBAL, _workspace=ws, _epoch=0)
+    assert ops._fused_workspace_status(ws) == 0
+    assert _mismatches(out, want[0])[0] == 0 and _mismatches(fin, want[1])[0] == 0
+    print("[promise] epoch 4 behind epoch 1, epoch 5 behind epoch 1", flush=True)
+    run(big, _kernel=GLOBAL, _workspace=ws, _epoch=4, _spin_limit=64)       # parity of a launch nobody made: its counters are zero
+    assert ops._fused_workspace_status(ws) == -10
+    run(big, _kernel=GLOBAL, _workspace=ws, _epoch=0)
+    run(big, _kernel=GLOBAL, _workspace=ws, _epoch=3, _spin_limit=64)       # same parity as epoch 1: its counters are used up
+    assert ops._fused_workspace_status(ws) == -10
+    # the wrappers' own workspace: small call, then the memory behind its flags poisoned with the next epoch, then the
+    # larger call -- which must clear again by itself
+    ops.release_workspaces()
+    run(small, _kernel=GLOBAL)
+    assert ops.fused_status() == 0
+    (kept,) = [k for key, k in ops_module._WORKSPACES.items() if key[0] == torch.cuda.current_device()]
+    kept.tensor[128 + 256:].fill_(2)
+    out, fin = run(big, _kernel=GLOBAL)
+    assert ops.fused_status() == 0
+    assert _mismatches(out, want[0])[0] == 0 and _mismatches(fin, want[1])[0] == 0
+    out, fin = run(big, _kernel=GLOBAL)                         # and goes on with epochs from there
+    assert ops.fused_status() == 0 and kept.epochs.last == 2
+    assert _mismatches(out, want[0])[0] == 0 and _mismatches(fin, want[1])[0] == 0
+
+
+def test_chain_failures_reach_the_caller_of_the_plain_wrappers(ops, oracle):
+    """The drop-in wrappers keep their workspace to themselves; fused_status() is how their caller learns that the last
+    launch failed.  One poll allowed: waves give up (and still raise their flags, so the launch drains) -> -7; the next
+    call is clean."""
+    d = oracle.make_inputs(1, b=1, L=8192, H=8)
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    ops.release_workspaces()
+    assert ops.fused_status() == 0                              # nothing kept yet
+    ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, _kernel=GLOBAL, _chunks_per_item=1, _spin_limit=1)
+    assert ops.fused_status() == -7
+    out, fin = ops._fused_chunk_state_state_passing_fwd_concurrent(*args, torch.float32)
+    assert ops.fused_status() == 0
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"])
+    assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+def test_chain_reports_xcds_that_are_not_what_it_assumed(ops, oracle):
+    """LOCAL deals the units to one ticket counter per XCD and relies on a workgroup of every XCD showing up.  With the
+    test hook the library is told a wrong number of XCDs: 4 makes pairs of XCDs share a counter (SSD_ERR_CHAIN_XCD), 16
+    leaves half of the counters without any workgroup, so their units are never computed (SSD_ERR_CHAIN_INCOMPLETE --
+    no error bit is set by anybody, the ticket counters tell).  Waits are short, every kernel exits normally."""
+    d = oracle.make_inputs(2, b=2, L=4096, H=16)                # 16 units x 16 chunks
+    args = [_dev(d[k]) for k in ("B", "x", "dt", "dA_cumsum")]
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    ws = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+    run = lambda **kw: ops._fused_chunk_state_state_passing_fwd(*args, torch.float32, initial_states=_dev(d["initial_states"]),
+                                                                _kernel=LOCAL, _chunks_per_item=2, _workspace=ws, **kw)
+    try:
+        for xcds, code in ((4, -8), (16, -9)):
+            print(f"[xcds] told {xcds}", flush=True)
+            assert ops.set_chain_xcds(xcds) in (0, 4)
+            run(_spin_limit=16)
+            assert ops._fused_workspace_status(ws) == code
+    finally:
+        ops.set_chain_xcds(0)
+    out, fin = run()
+    assert ops._fused_workspace_status(ws) == 0
+    assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+def test_chain_with_an_out_view_that_shares_cache_lines_between_tiles(ops, oracle):
+    """The per-XCD variant reads passed states back with plain loads, which is only safe while no two state tiles share
+    a 128-byte line.  A C-ABI caller may hand over an `out` that starts 16 bytes into an allocation: the call must still
+    be right (the library then exchanges the states through memory, whatever variant was asked for)."""
+    import ctypes
+    from ssd_amd import _lib
+    lib = _lib.load()
+    d = oracle.make_inputs(2, b=2, L=2048, H=32)                # 32 units: the library's own choice is the per-XCD variant
+    want_out, want_fin = oracle.fused_ref(d["B"], d["x"], d["dt"], d["dA_cumsum"], initial_states=d["initial_states"])
+    x, B, dt, dA, init = (_dev(d[k]) for k in ("x", "B", "dt", "dA_cumsum", "initial_states"))
+    b, L, H, P = x.shape
+    C, Q, N = dt.shape[2], dt.shape[3], B.shape[-1]
+    dims = _lib.dims_arg(b, L, H, P, N, 1, Q, C)
+    ws = torch.full((1 << 16,), -1, dtype=torch.int32, device="cuda")
+    for kernel in (LOCAL, 1):
+        buf = torch.full((b * C * H * P * N + 4,), float("nan"), device="cuda")
+        out = buf[4:].view(b, C, H, P, N)
+        assert out.data_ptr() % 128 == 16
+        fin = torch.full((b, H, P, N), float("nan"), device="cuda")
+        used = ctypes.c_int32(0)
+        opts = _lib.SsdFusedOpts(ws.data_ptr(), ws.numel() * 4, 0, kernel, 0, 0, ctypes.pointer(used))
+        T = _lib.tensor_arg
+        print(f"[out view] kernel={kernel}", flush=True)
+        rc = lib.ssd_fused_chunk_state_passing_fwd_ws(T(x), T(B), T(dt), T(dA), T(None), T(init), T(None), T(out), T(fin), dims, 1,
+                                                      ctypes.byref(opts), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0 and used.value == 1
+        assert ops._fused_workspace_status(ws) == 0
+        assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
