@@ -152,7 +152,12 @@ def main():
         return wall / steps, e0.elapsed_time(e1) * 1e-3 / steps     # seconds per step (host clock, device events)
 
     wall_step, ev_step = timed(fused, args.steps, args.warmup)
-    unf_wall, unf_ev = timed(unfused, max(5, args.steps // 4), 3)
+    # a failed chain (a wait that ran out, an XCD without a workgroup ...) leaves outputs unusable and says so only here
+    chain_status = ssd_amd.fused_status()
+    assert chain_status == 0, f"the fused launches report status {chain_status}"
+    # every figure beside the headline is an average over at least 20 launches, whatever --steps is
+    steps_2nd = max(20, args.steps // 4)
+    unf_wall, unf_ev = timed(unfused, steps_2nd, 3)
 
     # neighbours of the path, reported beside the headline: the fused call with bf16 passed states (what the
     # reference's main.py asks for, out_dtype = C.dtype) and the producer of dt / dA_cumsum
@@ -194,16 +199,39 @@ def main():
     def plain_copy(i):
         cp_dst[i % nsets].copy_(cp_src[i % nsets])
 
-    _, copy_ev = timed(plain_copy, max(5, args.steps // 4), 3)
+    _, copy_ev = timed(plain_copy, steps_2nd, 3)
     del cp_src, cp_dst
-    _, bf16_ev = timed(fused_bf16, max(5, args.steps // 4), 3)
-    _, cs_ev = timed(cumsum, max(5, args.steps // 4), 3)
-    _, prep_ev = timed(prep_fused, max(5, args.steps // 4), 3)
-    _, scan_ev = timed(scan_states, max(5, args.steps // 4), 3)
+
+    # ... and a kernel with this path's own streams and nothing else: x and B rows in, one fp32 state tile per (state
+    # tile, chunk) out, no arithmetic, no chain (ssd_measure_traffic_floor; it overwrites the `out` it is given)
+    mover_ev = None
+    if cfg["dtype"] == "bf16" and not args.with_states:
+        mv_out = [torch.empty(b, C, H, P, N, device=dev) for _ in range(nsets)]
+        mv_fin = torch.empty(b, H, P, N, device=dev)
+
+        def mover(i):
+            s = sets[i % nsets]
+            ssd_amd.measure_traffic_floor(s["B"], s["x"], s["dt"], s["dA_cumsum"], mv_out[i % nsets], mv_fin)
+
+        try:
+            _, mover_ev = timed(mover, steps_2nd, 3)
+        except RuntimeError as e:          # a shape the chain kernel does not cover has no such floor
+            log(f"[bench] no traffic floor for this workload: {e}")
+        del mv_out, mv_fin
+    _, bf16_ev = timed(fused_bf16, steps_2nd, 3)
+    _, cs_ev = timed(cumsum, steps_2nd, 3)
+    _, prep_ev = timed(prep_fused, steps_2nd, 3)
+    _, scan_ev = timed(scan_states, steps_2nd, 3)
     # ... and on bf16 passed states (the reference's main.py hands its scan `out` in C's type)
     prev_states = [fused_bf16(i)[0] for i in range(nsets)]
-    _, scan16_ev = timed(scan_states, max(5, args.steps // 4), 3)
+    _, scan16_ev = timed(scan_states, steps_2nd, 3)
     del prev_states, y_bufs
+    # the headline call again without the clock ramp, right after host-side idling: what a lone call in a quiet stream sees
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    saved_ramp, args.ramp_ms = args.ramp_ms, 0.0
+    _, cold_ev = timed(fused, 20, 0)
+    args.ramp_ms = saved_ramp
 
     # parity of what was timed, over the whole batch, against the CPU oracle (the long grouped configuration on four
     # heads of different groups: its fp32 oracle would not fit a few minutes)
@@ -226,8 +254,6 @@ def main():
     torch.cuda.synchronize()
     bad, worst, scope = parity(args.config, d, out, fin)
     log(f"[bench] parity ({scope}): max|err|={worst:.3e}, mismatches={bad}")
-    sl = slice(0, 1)
-    cut = lambda t: None if t is None else t[sl]
     del out, fin
 
     alg_bytes = ssd_oracle.algorithmic_bytes(cfg, with_states=args.with_states)
@@ -258,7 +284,11 @@ def main():
                                        + kernel_source_hash() + " (null: not measured on these sources)",
                      "algorithmic_bytes": alg_bytes, "kernel_us": round(ev_step * 1e6, 2),
                      "plain_copy_us": round(copy_ev * 1e6, 2), "plain_copy_gbps": round(2 * half / copy_ev / 1e9, 1),
-                     "frac_of_plain_copy": round(copy_ev * 2 * half / alg_bytes / ev_step, 4)},
+                     "frac_of_plain_copy": round(copy_ev * 2 * half / alg_bytes / ev_step, 4),
+                     "mover_us": None if mover_ev is None else round(mover_ev * 1e6, 2),
+                     "mover_bytes": None if mover_ev is None else b * L * H * P * 2 + d["B"].numel() * 2 + b * C * H * P * N * 4,
+                     "frac_of_mover": None if mover_ev is None else round(mover_ev / ev_step, 4),
+                     "kernel_us_cold": round(cold_ev * 1e6, 2), "frac_cold": round(alg_bytes / cold_ev / 1e9 / HBM_PEAK_GBPS, 4)},
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "unfused_us": round(unf_ev * 1e6, 2),
@@ -275,7 +305,7 @@ def main():
     if not args.no_per_config:
         # the same call, timed the same way, on each of the five configurations
         table = {}
-        steps_pc = max(5, args.steps // 4)
+        steps_pc = steps_2nd
         for idx in range(5):
             c = ssd_oracle.CONFIGS[idx]
             if idx == args.config:
@@ -310,21 +340,29 @@ def main():
         res["per_config"] = table
 
     if not args.no_cpu:
-        # reference math in fp32 PyTorch on this machine's host cores: one batch row of the workload
-        # (a bounded sample), scaled to the full layer
+        # reference math in fp32 PyTorch on this machine's host cores: the whole batch of the workload, one warm-up
+        # and three timed repetitions (the long grouped configuration: one repetition on 8 of its 128 heads, scaled)
         nthreads = torch.get_num_threads()
-        args_cpu = (d["B"][sl], d["x"][sl], d["dt"][sl], d["dA_cumsum"][sl])
-        kw_cpu = dict(initial_states=cut(d["initial_states"]), seq_idx=cut(d["seq_idx"]))
-        ssd_oracle.fused_ref(*args_cpu, **kw_cpu)
+        if args.config == 4:
+            hs, scale, reps = slice(0, 8), H / 8, 1
+            args_cpu = (d["B"][:, :, 0:1], d["x"][:, :, hs], d["dt"][:, hs], d["dA_cumsum"][:, hs])
+            what = f"heads 0-7 of {H}, 1 repetition, scaled x{H // 8}"
+        else:
+            scale, reps = 1.0, 3
+            args_cpu = (d["B"], d["x"], d["dt"], d["dA_cumsum"])
+            what = "the whole batch, 1 warm-up + 3 repetitions, median"
+        kw_cpu = dict(initial_states=d["initial_states"] if args.config != 4 else None, seq_idx=d["seq_idx"])
+        if reps > 1:
+            ssd_oracle.fused_ref(*args_cpu, **kw_cpu)
         ts = []
-        for _ in range(2):
+        for _ in range(reps):
             t0 = time.perf_counter()
             ssd_oracle.fused_ref(*args_cpu, **kw_cpu)
             ts.append(time.perf_counter() - t0)
-        cpu_s = sorted(ts)[0] * b
+        cpu_s = sorted(ts)[len(ts) // 2] * scale
         res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us/layer", "cores": nthreads, "kind": "port",
-                               "sample": f"fp32 PyTorch restatement of the reference math (oracle/ssd_oracle.py fused_ref) on batch "
-                                         f"row 0 of {b}, best of 2, scaled x{b}; torch threads={nthreads}, os.cpu_count()={os.cpu_count()}"}
+                               "sample": f"fp32 PyTorch restatement of the reference math (oracle/ssd_oracle.py fused_ref) on {what}; "
+                                         f"torch threads={nthreads}, os.cpu_count()={os.cpu_count()}"}
     print(json.dumps(res), flush=True)
 
 

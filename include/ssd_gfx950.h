@@ -354,6 +354,19 @@ int ssd_set_scan_kernel(int kernel);
 int ssd_set_token_split(int waves);
 
 /*
+ * Measurement hook with no counterpart in the reference: the memory traffic of the fused call on these tensors with
+ * all arithmetic, all dependencies between chunks and all waiting on other workgroups removed -- every x row read
+ * once, every B row once per four state tiles, one 32 x dstate fp32 tile written per (state tile, chunk), by one
+ * persistent workgroup per compute unit with the fused kernels' request and store patterns.  Its duration is the floor
+ * the memory system of the device sets for the path's access pattern (bench.py reports it as roofline.mover_us next to
+ * the fused call's time).  dt, dA_cumsum and final_states are only checked, not moved (6 % of the path's bytes).
+ * `out` IS OVERWRITTEN (with zeros).  Arguments the ticket / flag-chain kernel does not cover (it needs bf16 x / B,
+ * fp32 out, dstate 64 or 128, chunk 128 or 256, four state tiles per (batch, group)): SSD_ERR_SHAPE.
+ */
+int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                              const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, void *stream);
+
+/*
  * Test hook with no counterpart in the reference: the number of XCDs (L2 caches) the LOCAL variant of the ticket /
  * flag-chain kernel deals its units to; 0 = compute units / 32 (the default; 8 on MI355X), at most 16.  A wrong count
  * is what the kernel's own checks exist for (SSD_ERR_CHAIN_XCD, SSD_ERR_CHAIN_INCOMPLETE) and how the tests provoke

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libssd_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
-SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_chain.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip"]
+SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_chain.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # keep the compiler from forming packed-fp32 VALU instructions

@@ -695,6 +695,19 @@ int ssd_set_scan_kernel(int kernel)
     return ssd::set_scan_kernel(kernel);
 }
 
+int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                              const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, void *stream)
+{
+    Params p;
+    int rc = fill_fused(p, x, B, dt, dA_cumsum, nullptr, nullptr, nullptr, out, final_states, dims, 1);
+    if (rc) return rc;
+    if (!ssd::chain_supported(p) || p.dt_out != ssd::DT_F32) return SSD_ERR_SHAPE;
+    rc = check_device();
+    if (rc) return rc;
+    const int n_cu = compute_units();
+    return (int)ssd::launch_mover(p, n_cu > 0 ? n_cu : 256, (hipStream_t)stream);
+}
+
 int ssd_set_chain_xcds(int xcds)
 {
     if (xcds < 0 || xcds > ssd::kChainMaxXcd) return SSD_ERR_SHAPE;

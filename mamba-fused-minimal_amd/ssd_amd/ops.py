@@ -485,6 +485,22 @@ def set_scan_kernel(kernel):
     return rc
 
 
+def measure_traffic_floor(B, x, dt, dA_cumsum, out, final_states):
+    """Measurement hook (no counterpart in the reference): enqueues the kernel that moves the bytes of the fused call on
+    these tensors -- x and B read, one fp32 state tile per (state tile, chunk) written -- and does nothing else
+    (ssd_measure_traffic_floor).  ``out`` (b,C,H,P,N) fp32 is overwritten with zeros."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert out.shape == (batch, nchunks, nheads, headdim, dstate) and final_states.shape == (batch, nheads, headdim, dstate)
+    _lib.require_device(x, "measure_traffic_floor")
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    T = _lib.tensor_arg
+    with torch.cuda.device(x.device):
+        rc = _lib.load().ssd_measure_traffic_floor(T(x), T(B), T(dt), T(dA_cumsum), T(out), T(final_states), dims, _stream(x))
+    _lib.check(rc, "ssd_measure_traffic_floor")
+
+
 def set_chain_xcds(xcds):
     """Test hook (no counterpart in the reference): the number of XCDs the per-XCD variant of the ticket / flag-chain
     kernel deals its units to; 0 = from the device.  A wrong count provokes the kernel's own checks

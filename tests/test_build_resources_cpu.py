@@ -34,7 +34,7 @@ def test_every_source_reports_its_kernels(usage):
     counts = {src: len(kernels) for src, kernels in usage.items()}
     assert counts["ssd_capi.hip"] == 0                       # host code only
     for src in ("ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_generic.hip", "ssd_state_passing.hip",
-                "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip"):
+                "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip"):
         assert counts[src] > 0, src
     # the chain kernel: dstate 64 / 128 x chunk 128 / 256 x 1 / 2 / 4 chunks per item (2 / 4 with bf16 out) x seq_idx or
     # not x LOCAL / GLOBAL, + the fill

@@ -510,3 +510,25 @@ def test_chain_with_an_out_view_that_shares_cache_lines_between_tiles(ops, oracl
         assert rc == 0 and used.value == 1
         assert ops._fused_workspace_status(ws) == 0
         assert _mismatches(out, want_out)[0] == 0 and _mismatches(fin, want_fin)[0] == 0
+
+
+@pytest.mark.parametrize("kw", [dict(b=2, L=2048, H=8), dict(L=2000, H=8), dict(Q=128, L=1408, N=64, H=8), dict(P=128, H=4, G=2, L=1280)],
+                         ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))
+def test_traffic_floor_kernel_covers_every_output_tile(ops, oracle, kw):
+    """ssd_measure_traffic_floor moves the fused call's bytes and computes nothing; bench.py prices the fused kernels
+    against its duration.  What can be checked of it: it writes every element of `out` (here NaN before, zero after --
+    a tile it skipped would make the floor too low) and touches nothing else."""
+    base = dict(b=2, L=1024, H=6, G=1)
+    base.update(kw)
+    d = oracle.make_inputs(1, **base)
+    x, B, dt, dA = (_dev(d[k]) for k in ("x", "B", "dt", "dA_cumsum"))
+    b, L, H, P = x.shape
+    C, N = dt.shape[2], B.shape[-1]
+    out = torch.full((b, C, H, P, N), float("nan"), device="cuda")
+    fin = torch.full((b, H, P, N), float("nan"), device="cuda")
+    ops.measure_traffic_floor(B, x, dt, dA, out, fin)
+    torch.cuda.synchronize()
+    assert int((out != 0).sum()) == 0
+    assert bool(torch.isnan(fin).all())
+    with pytest.raises(RuntimeError):                      # fp32 inputs are not the chain kernel's: no floor defined
+        ops.measure_traffic_floor(B.float(), x.float(), dt, dA, out, fin)
