@@ -45,11 +45,14 @@ using namespace tile;
 // compute unit leaves the room, and the burst of state stores that ends an item drains behind requests that far
 // ahead -- else 4
 template <int SPC> constexpr int ring_of() { return SPC >= 8 ? 8 : 4; }
+// B rows are read by every head of a group and come from L2 after the first reader: three steps ahead cover that
+// latency, and the four-step ring leaves LDS to others
+constexpr int kRingB = 4, kDistB = kRingB - 1;
 // per wave: x ring + two weight slots (the next item's weights are written while the current item's are in use)
 template <int SPC> constexpr int wave_lds() { return ring_of<SPC>() * 2048 + 2 * 32 * SPC * 4; }
 constexpr int kStage = 1024;        // per wave: a 16 x 16 fp32 block of the state on its way to or from memory
 constexpr int kTicketBytes = 64;
-template <int NT, int SPC> constexpr int lds_bytes() { return ring_of<SPC>() * NT * 1024 + 4 * (wave_lds<SPC>() + kStage) + kTicketBytes; }
+template <int NT, int SPC> constexpr int lds_bytes() { return kRingB * NT * 1024 + 4 * (wave_lds<SPC>() + kStage) + kTicketBytes; }
 
 // How the passed states cross between compute units.  The L2 caches, one per XCD (32 compute units), are not
 // coherent with each other, and a device-scope release / acquire pair writes back and invalidates a whole L2
@@ -82,17 +85,17 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     static_assert(kDist < SPC, "the requests of a step reach into the next chunk at most");
     // the step loop's vector-memory queue, replayed at compile time (ssd_tile.h): 2 x requests and NT / 4 B requests
     // per step, no stores inside the loop
-    constexpr schedule::Loop kLoop{2, NT / 4, 0, SPC, kDist, kRing};
+    constexpr schedule::Loop kLoop{2, NT / 4, 0, SPC, kDist, kRing, kDistB};
     static_assert(schedule::slots_ok(kLoop), "ring slots are reused too early");
     constexpr int TPL = Q / 64;         // tokens per lane when an item's weights are computed (2 or 4)
     constexpr int NTW = NT / 4;         // B tile blocks (32 tokens x 16 columns, 1 KB) a wave fetches per step
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int lane = threadIdx.x & 63, i16 = lane & 15, kg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    char *bring = lds;                                                   // kRing x NT blocks of 1 KB, shared
-    char *xring = lds + kRing * NT * 1024 + wave * wave_lds<SPC>();      // kRing slots x (32 tokens x 64 bytes)
+    char *bring = lds;                                                   // kRingB x NT blocks of 1 KB, shared
+    char *xring = lds + kRingB * NT * 1024 + wave * wave_lds<SPC>();     // kRing slots x (32 tokens x 64 bytes)
     char *wbuf = xring + kRing * 2048;                                   // 2 slots x Q weights
-    char *stage = lds + kRing * NT * 1024 + 4 * wave_lds<SPC>() + wave * kStage;
+    char *stage = lds + kRingB * NT * 1024 + 4 * wave_lds<SPC>() + wave * kStage;
 #if defined(__HIP_DEVICE_COMPILE__)      // typed as LDS: a volatile access through a generic pointer would go the flat way
     typedef __attribute__((address_space(3))) volatile int lds_int;
     lds_int *tq = (lds_int *)(__attribute__((address_space(3))) char *)(lds + lds_bytes<NT, SPC>() - kTicketBytes);
@@ -186,7 +189,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 #if defined(__HIP_DEVICE_COMPILE__)      // the LDS address space does not exist in the host pass
         typedef __attribute__((address_space(3))) void *lds_ptr;
         const int th = bi / (NT / 2), pair = bi % (NT / 2);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRing) * NT + bi) * 1024), 16, Blane,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(bring + ((s % kRingB) * NT + bi) * 1024), 16, Blane,
                                                  (int)((32 * s + 16 * th) * Brb) + 64 * pair, 0, 0);
 #else
         (void)rs; (void)s; (void)bi; (void)Blane;
@@ -534,7 +537,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 #pragma unroll
     for (int i = 0; i < 2 * kRing; ++i) *(u32x4 *)(xring + i * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < kRing * NTW; ++i)
+    for (int i = 0; i < kRingB * NTW; ++i)
         *(u32x4 *)(bring + (i * 4 + wave) * 1024 + 16 * lane) = (u32x4){0u, 0u, 0u, 0u};
     __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): the zeros are in place before any row lands
     __builtin_amdgcn_s_barrier();
@@ -556,12 +559,15 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     }
 
     Meta mcur = load_meta(cur);
-    // requests of the steps 0..kDist-1, in the order (x, x, B...) that every later step keeps
+    // requests of the steps 0..kDist-1 (B: 0..kDistB-1), in the order (x, x, B...) that every later step keeps
 #pragma unroll
     for (int s = 0; s < kDist; ++s) {
         load_x(cur.rsx, cur.p0, s, 0); load_x(cur.rsx, cur.p0, s, 1);
+        // (beyond the B distance: requests with an empty descriptor, which fetch nothing -- they keep the number of
+        // operations per step, which the waits below count, the same from the first step on.  What such a request
+        // deposits is zeros, so it is aimed at the one ring slot no real request has been made for yet.)
 #pragma unroll
-        for (int k = 0; k < NTW; ++k) load_B(cur.rsB, s, wave * NTW + k);
+        for (int k = 0; k < NTW; ++k) load_B(s < kDistB ? cur.rsB : make_rsrc(nullptr, 0), s < kDistB ? s : kDistB, wave * NTW + k);
         __builtin_amdgcn_sched_barrier(0);
     }
     put_weights(cur.c, 0, mcur);
@@ -570,12 +576,12 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
     // boundaries: block t of the stream of (step, tile) pairs sits in slot t % 4
     constexpr int kAhead = 3;
     static_assert(NT % 4 == 0 && kAhead < 4 && kAhead <= NT, "slot of a block = its tile index % 4");
-    static_assert(SPC % kRing == 0, "ring slots repeat from item to item");
+    static_assert(SPC % kRing == 0 && SPC % kRingB == 0, "ring slots repeat from item to item");
     u32x2 blo[4], bhi[4];
     {
-        // everything up to this wave's B blocks of step 0 has landed: the requests of two steps were issued later
+        // everything up to this wave's B blocks of step 0 has landed: the requests of the other steps were issued later
         static_assert(schedule::wait_prologue(kLoop) == (kDist - 1) * (2 + NTW), "prologue wait");
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 1) * (2 + NTW)));
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(schedule::wait_prologue(kLoop)));
         __builtin_amdgcn_s_barrier();   // ... and every other wave's blocks of step 0
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
@@ -614,11 +620,11 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         // published by this step's barrier: the ticket after next, or (first item) the next one and then that
         if (s == SPC - 2 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
             tq[second_late && cur.r == 0 ? 1 : 2] = t_new;
-        // requests of this step: x rows and this wave's B blocks of step + 3 (this item or the next)
-        const auto rsB = s + kDist < SPC ? cur.rsB : nxt.rsB;
+        // requests of this step: x rows of step + kDist and this wave's B blocks of step + kDistB (this item or the next)
+        const auto rsB = s + kDistB < SPC ? cur.rsB : nxt.rsB;
         const auto rsx = s + kDist < SPC ? cur.rsx : nxt.rsx;
         const int xp0 = s + kDist < SPC ? cur.p0 : nxt.p0;
-        const int s3 = (s + kDist) % SPC;
+        const int s3 = (s + kDist) % SPC, s3b = (s + kDistB) % SPC;
         const bf16x8 h0 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[0][0], fc.hi[0][1], fc.hi[0][2], fc.hi[0][3]});
         const bf16x8 h1 = __builtin_bit_cast(bf16x8, (u32x4){fc.hi[1][0], fc.hi[1][1], fc.hi[1][2], fc.hi[1][3]});
         const bf16x8 l0 = __builtin_bit_cast(bf16x8, (u32x4){fc.lo[0][0], fc.lo[0][1], fc.lo[0][2], fc.lo[0][3]});
@@ -634,14 +640,14 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 // ago) have landed once only the requests of step - 1 and the x requests of this step are
                 // outstanding; the barrier publishes every wave's blocks.  It also tells that all waves are through
                 // with the tile of step - 1, whose ring slot the B requests below overwrite.
-                static_assert(schedule::wait_b(kLoop, s) == (kDist - 2) * (2 + NTW) + 2, "wait for the B blocks of step + 1");
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm((kDist - 2) * (2 + NTW) + 2));
+                static_assert(schedule::wait_b(kLoop, s) == (kDistB - 2) * (2 + NTW) + 2, "wait for the B blocks of step + 1");
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(schedule::wait_b(kLoop, s)));
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             }
             {
                 constexpr int tn = it + kAhead;     // block kAhead iterations on: this step's tile or the next one's
-                read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
+                read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRingB>{}, std::integral_constant<int, tn % NT>{},
                         blo[tn % 4], bhi[tn % 4]);
             }
             // a chunk's first step starts its sums: the accumulators are not cleared, the MFMA takes zero instead
@@ -658,7 +664,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 for (int e = e0; e < e1; ++e) frag_piece(e >> 1, e & 1, xr, wv, fn);
             }
             if (it == 0) { load_x(rsx, xp0, s3, 0); load_x(rsx, xp0, s3, 1); }
-            if (it >= NT - kAhead && it < NT - kAhead + NTW) load_B(rsB, s3, wave * NTW + (it - (NT - kAhead)));
+            if (it >= NT - kAhead && it < NT - kAhead + NTW) load_B(rsB, s3b, wave * NTW + (it - (NT - kAhead)));
             if (s == 1 && it == NT - 1 && nxt.valid) mnext = load_meta(nxt);
             __builtin_amdgcn_sched_barrier(0);
         });

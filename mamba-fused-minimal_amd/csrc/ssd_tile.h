@@ -75,7 +75,10 @@ __device__ __forceinline__ void store4_bf16(__amdgpu_buffer_rsrc_t rs, int voff,
 // inputs, tickets, a chain step -- are issued after X or complete before it, and only make a wait longer).
 namespace schedule {
 
-struct Loop { int xr, bw, st, spc, dist, ring; };    // st: stores at a chunk's first step (0 = none)
+// st: stores at a chunk's first step (0 = none); dist_b: the B requests' own distance where it is shorter than that
+// of the x requests (B rows come from L2 after their first reader, x rows from memory), -1 = the same
+struct Loop { int xr, bw, st, spc, dist, ring; int dist_b = -1; };
+constexpr int b_dist(Loop k) { return k.dist_b < 0 ? k.dist : k.dist_b; }
 constexpr int kSteps = 48;                           // steps replayed: several chunks past the prologue
 struct Waits { int w0; int w1[kSteps]; int w2[kSteps]; };
 
@@ -86,7 +89,8 @@ constexpr Waits replay(Loop k)
     int n = 0;      // operations issued so far
     for (int t = 0; t < k.dist; ++t) {
         n += k.xr; last_x[t] = n - 1;
-        n += k.bw; last_b[t] = n - 1;
+        n += k.bw;          // beyond the B distance these are requests that fetch nothing: every step issues the same number
+        if (t < b_dist(k)) last_b[t] = n - 1;
     }
     r.w0 = n - 1 - last_b[0];
     for (int t = 0; t < kSteps; ++t) {
@@ -94,7 +98,7 @@ constexpr Waits replay(Loop k)
         if (k.st > 0 && t % k.spc == 0) n += k.st;
         n += k.xr; last_x[t + k.dist] = n - 1;
         r.w2[t] = n - 1 - last_b[t + 1];
-        n += k.bw; last_b[t + k.dist] = n - 1;
+        n += k.bw; last_b[t + b_dist(k)] = n - 1;
     }
     return r;
 }
@@ -119,7 +123,12 @@ constexpr int wait_prologue(Loop k) { return replay(k).w0; }
 // wave has consumed the tile of step u by the end of step u, and the requests of step t follow that step's barrier,
 // so u < t.  Both hold with a ring one longer than the distance; requests must not reach past the next chunk, and
 // the slot of a step must not depend on the chunk.
-constexpr bool slots_ok(Loop k) { return k.ring == k.dist + 1 && k.dist < k.spc && k.spc % k.ring == 0 && k.spc <= kSteps / 3; }
+// (A B ring shorter than the x ring: one longer than the B distance, by the same argument.)
+constexpr bool slots_ok(Loop k)
+{
+    return k.ring == k.dist + 1 && k.dist < k.spc && k.spc % k.ring == 0 && k.spc <= kSteps / 3 && b_dist(k) <= k.dist &&
+           b_dist(k) >= 1 && k.spc % (b_dist(k) + 1) == 0;
+}
 
 }  // namespace schedule
 
