@@ -333,6 +333,34 @@ int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states
                               void *stream);
 
 /*
+ * Chunk state + state passing + the consumer above in ONE launch: the ticket / flag-chain kernel multiplies the state
+ * entering each chunk by that chunk's C rows in its chain step, while the state sits in registers, so the passed
+ * states need not reach memory at all.  Replaces kernels/fused_concurrent.py:255-331 (or fused_globalbar.py:201-266)
+ * followed by the state-dependent half of kernels/ssd_chunk_scan.py:94-117, as main.py:85-86 and :100-101 call them.
+ *   y[b,cQ+m,h,p] (+)= exp(dA_cumsum[b,h,c,m]) * [seq_idx[b,cQ+m] == seq_idx[b,cQ-1]] * sum_n C[b,cQ+m,g,n] * out[b,c,h,p,n]
+ * with out[:, c] the state entering chunk c exactly as ssd_fused_chunk_state_passing_fwd defines it -- in fp32, split
+ * into bf16 hi + lo for the matrix cores (the reference rounds it to C's element type, kernels/ssd_chunk_scan.py:106-110).
+ * Arguments of ssd_fused_chunk_state_passing_fwd_ws without `states`, plus C (batch, seqlen, ngroups, dstate; the
+ * element type of x) and y (batch, seqlen, nheads, headdim; fp32 or bf16, innermost stride 1); accumulate != 0 adds to
+ * what y holds.  `out` MAY BE ABSENT (out == NULL or out->data == NULL): then the only trace of the passed states is
+ * one 32 x dstate fp32 slot per (state tile, work item) in the workspace, and final_states.  opts: as in
+ * ssd_fused_chunk_state_passing_fwd_ws; the workspace must hold ssd_fused_scan_workspace_bytes(dims, with_out,
+ * opts->chunks_per_item) bytes, 16-byte aligned (with_out: `out` is given, fp32; work items are two chunks long with
+ * dstate 128 -- what the register file holds next to the operands of the second product -- and up to four with dstate 64).
+ * The one-launch kernel takes what the chain kernel takes (bf16 x / B / C, fp32 out if any, dstate 64 or 128, chunk 128
+ * or 256, four state tiles per (batch, group), 16-byte aligned rows) and needs the workspace.  Any other call WITH `out`
+ * runs as ssd_fused_chunk_state_passing_fwd[_ws] followed by ssd_chunk_scan_states_fwd (*opts->used_workspace says which
+ * happened); without `out` and without that kernel there is no place for the passed states: SSD_ERR_SCRATCH (the
+ * library never allocates).
+ */
+uint64_t ssd_fused_scan_workspace_bytes(const ssd_dims *dims, int with_out, int chunks_per_item);
+int ssd_fused_chunk_state_passing_scan_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *C, const ssd_tensor *dt,
+                                           const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                           const ssd_tensor *initial_states, const ssd_tensor *out,
+                                           const ssd_tensor *final_states, const ssd_tensor *y, const ssd_dims *dims,
+                                           int clamp, int accumulate, const ssd_fused_opts *opts, void *stream);
+
+/*
  * Tuning / test hook with no counterpart in the reference: which matrix-core kernel serves ssd_chunk_scan_states_fwd
  * where both apply.  0 = let the library choose (the default); 1 = one workgroup per (batch, chunk, head);
  * 2 = one workgroup per run of heads, with the chunk's C rows kept in LDS across the run (needs headdim % 64 == 0

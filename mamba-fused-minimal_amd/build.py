@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libssd_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
-SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_chain.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip"]
+SOURCES = ["ssd_capi.hip", "ssd_mfma.hip", "ssd_quad.hip", "ssd_chain.hip", "ssd_generic.hip", "ssd_state_passing.hip", "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip", "ssd_chain_scan.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # keep the compiler from forming packed-fp32 VALU instructions
@@ -21,6 +21,7 @@ FLAGS = [
     "-Rpass-analysis=kernel-resource-usage",
 ]
 USAGE = os.path.join(OBJ_DIR, "resource_usage.json")
+ISA_CHECK = os.path.join(OBJ_DIR, "async_operand_check.json")
 
 
 def hipcc():
@@ -69,16 +70,43 @@ def build_library(verbose=False, extra_flags=(), jobs=None):
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 8)
 
     def compile_one(src):
-        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc(), *compile_flags, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        # the compiler's intermediate files (the gfx950 assembly among them) go to a directory per source
+        stem = os.path.splitext(src)[0]
+        obj = os.path.join(OBJ_DIR, stem + ".o")
+        tmp = os.path.join(OBJ_DIR, "temps_" + stem)
+        shutil.rmtree(tmp, ignore_errors=True)
+        os.makedirs(tmp)
+        cmd = [hipcc(), *compile_flags, *extra_flags, "--save-temps", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd))
-        return obj, _run(cmd)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=tmp)
+        noise = "is not a recognized feature for this target"
+        out = "\n".join(l for l in res.stdout.splitlines() if noise not in l)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + out)
+        return obj, out
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(compile_one, SOURCES))
-    out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in results], "-o", LIB])
+    # the generated code, checked for copies of operands that inline assembly is still loading (isa_check.py)
+    sys.path.insert(0, HERE)
+    import isa_check
+    findings = {}
+    for src in SOURCES:
+        tmp = os.path.join(OBJ_DIR, "temps_" + os.path.splitext(src)[0])
+        for name in sorted(os.listdir(tmp)):
+            if name.endswith("gfx950.s"):
+                findings[src] = isa_check.check_file(os.path.join(tmp, name))
+        shutil.rmtree(tmp, ignore_errors=True)
     import json
+    with open(ISA_CHECK, "w") as f:
+        json.dump(findings, f, indent=1, sort_keys=True)
+    bad = {k: v for k, v in findings.items() if v}
+    if bad:
+        first = next(iter(bad.values()))[0]
+        raise RuntimeError(f"the compiler moved operands that inline assembly is still loading in {sorted(bad)} "
+                           f"({sum(len(v) for v in bad.values())} places, e.g. {first}); see {ISA_CHECK}")
+    out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in results], "-o", LIB])
     usage = {}
     for src, (_, text) in zip(SOURCES, results):
         usage[src], rest = _resource_usage(text)

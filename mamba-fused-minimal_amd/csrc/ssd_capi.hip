@@ -290,17 +290,18 @@ int chain_decision(const Params &p, const ssd_dims *dims, const ssd_fused_opts *
     if (opts && opts->used_workspace) *opts->used_workspace = 0;
     const int kernel = opts ? opts->kernel : SSD_KERNEL_AUTO;
     if (kernel < SSD_KERNEL_AUTO || kernel > SSD_KERNEL_CHAIN_GLOBAL) return SSD_ERR_SHAPE;
-    // bf16 out: the workspace also holds the fp32 states that cross between items, as many as the launch will have
-    // items (the forced number of chunks per item, or the one the launch would choose)
-    const bool out16 = p.dt_out != ssd::DT_F32;
+    // bf16 out (or none): the workspace also holds the fp32 states that cross between items, as many as the launch will
+    // have items (the forced number of chunks per item, or the one the launch would choose)
+    const bool out16 = ssd::chain_needs_carry(p);
     const int forced_r = opts ? opts->chunks_per_item : 0;
     const int r = out16 ? ssd::chain_chunks_per_item(p, compute_units(), forced_r) : 0;
     const uint64_t need = out16 ? ssd::chain_workspace_bytes_out16(dims->batch, dims->nheads, dims->headdim, dims->dstate, dims->nchunks, r)
                                 : ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
     const bool have_ws = opts && opts->workspace && ((uintptr_t)opts->workspace % (out16 ? 16 : 4)) == 0 &&
                          opts->workspace_bytes >= need && !(out16 && r < 2);
+    // with the scan's state half asked for, the chain kernel is the only one that computes it in the same launch
     if (have_ws && ssd::chain_supported(p) &&
-        (kernel != SSD_KERNEL_AUTO || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
+        (kernel != SSD_KERNEL_AUTO || p.y || (g_forced_split.load(std::memory_order_relaxed) == 0 && chain_preferred(p, compute_units())))) {
         *use = true;
         if (opts->used_workspace) *opts->used_workspace = 1;
         return check_device();
@@ -383,18 +384,23 @@ int ssd_chunk_state_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tens
     return run(p, false, stream);
 }
 
-// Fills Params for a fused call (chunk state + state passing).
+// Fills Params for a fused call (chunk state + state passing).  out_optional: `out` may be absent.
 static int fill_fused(Params &p, const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
                       const ssd_tensor *seq_idx, const ssd_tensor *initial_states, const ssd_tensor *states,
-                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, int clamp)
+                      const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, int clamp,
+                      bool out_optional = false)
 {
-    if (!present(out) || !present(final_states)) return SSD_ERR_NULL;
+    if ((!present(out) && !out_optional) || !present(final_states)) return SSD_ERR_NULL;
     int rc = fill_common(p, x, B, dt, dA_cumsum, seq_idx, states, dims, clamp);
     if (rc) return rc;
-    if (!dtype_ok(out->dtype) || final_states->dtype != SSD_F32) return SSD_ERR_DTYPE;
-    if (out->stride[4] != 1 || final_states->stride[3] != 1) return SSD_ERR_STRIDE;
-    p.out = out->data; p.dt_out = out->dtype;
-    p.so_b = out->stride[0]; p.so_c = out->stride[1]; p.so_h = out->stride[2]; p.so_p = out->stride[3];
+    if (final_states->dtype != SSD_F32) return SSD_ERR_DTYPE;
+    if (final_states->stride[3] != 1) return SSD_ERR_STRIDE;
+    if (present(out)) {
+        if (!dtype_ok(out->dtype)) return SSD_ERR_DTYPE;
+        if (out->stride[4] != 1) return SSD_ERR_STRIDE;
+        p.out = out->data; p.dt_out = out->dtype;
+        p.so_b = out->stride[0]; p.so_c = out->stride[1]; p.so_h = out->stride[2]; p.so_p = out->stride[3];
+    }
     p.fin = (float *)final_states->data;
     p.sf_b = final_states->stride[0]; p.sf_h = final_states->stride[1]; p.sf_p = final_states->stride[2];
     if (present(initial_states)) {
@@ -651,6 +657,57 @@ int ssd_chunk_cumsum_fwd(const ssd_tensor *dt, const ssd_tensor *A, const ssd_te
     rc = check_device();
     if (rc) return rc;
     return (int)ssd::launch_chunk_cumsum(p, (hipStream_t)stream);
+}
+
+uint64_t ssd_fused_scan_workspace_bytes(const ssd_dims *dims, int with_out, int chunks_per_item)
+{
+    if (check_dims(dims)) return 0;
+    if (with_out) return ssd::chain_workspace_bytes(dims->batch, dims->nheads, dims->headdim, dims->nchunks);
+    Params p;
+    memset(&p, 0, sizeof(p));
+    p.batch = dims->batch; p.nheads = dims->nheads; p.headdim = dims->headdim; p.dstate = dims->dstate;
+    p.C = dims->nchunks; p.Q = dims->chunk_size; p.y = (void *)16;
+    const int r = ssd::chain_chunks_per_item(p, compute_units(), chunks_per_item);
+    return ssd::chain_workspace_bytes_out16(dims->batch, dims->nheads, dims->headdim, dims->dstate, dims->nchunks, r);
+}
+
+int ssd_fused_chunk_state_passing_scan_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *C, const ssd_tensor *dt,
+                                           const ssd_tensor *dA_cumsum, const ssd_tensor *seq_idx,
+                                           const ssd_tensor *initial_states, const ssd_tensor *out,
+                                           const ssd_tensor *final_states, const ssd_tensor *y, const ssd_dims *dims,
+                                           int clamp, int accumulate, const ssd_fused_opts *opts, void *stream)
+{
+    if (!present(C) || !present(y)) return SSD_ERR_NULL;
+    Params p;
+    int rc = fill_fused(p, x, B, dt, dA_cumsum, seq_idx, initial_states, nullptr, out, final_states, dims, clamp, true);
+    if (rc) return rc;
+    if (!dtype_ok(C->dtype) || !dtype_ok(y->dtype)) return SSD_ERR_DTYPE;
+    if (C->stride[3] != 1 || y->stride[3] != 1) return SSD_ERR_STRIDE;
+    Params q = p;
+    q.Cm = C->data; q.sC_b = C->stride[0]; q.sC_l = C->stride[1]; q.sC_g = C->stride[2];
+    q.y = y->data; q.dt_y = y->dtype; q.sy_b = y->stride[0]; q.sy_l = y->stride[1]; q.sy_h = y->stride[2];
+    q.y_accumulate = accumulate ? 1 : 0;
+    if (q.batch == 1) q.sC_b = q.sy_b = 0;
+    if (q.ngroups == 1) q.sC_g = 0;
+    if (q.nheads == 1) q.sy_h = 0;
+    bool chain = false;
+    if (C->dtype == x->dtype) {
+        rc = chain_decision(q, dims, opts, &chain);
+        if (rc && present(out)) { rc = SSD_OK; chain = false; }      // forced, but not possible: the two calls below still are
+        if (rc) return rc;
+    } else if (opts && opts->used_workspace) {
+        *opts->used_workspace = 0;
+    }
+    if (chain) return run_chain(q, opts, stream);
+    // Elsewhere the passed states have to exist in memory: the fused call as it would run without y, then the
+    // stand-alone consumer over its `out`.
+    if (!present(out)) return SSD_ERR_SCRATCH;
+    bool plain_chain = false;
+    rc = chain_decision(p, dims, opts, &plain_chain);
+    if (rc) { rc = SSD_OK; plain_chain = false; }
+    rc = plain_chain ? run_chain(p, opts, stream) : run(p, true, stream);
+    if (rc) return rc;
+    return ssd_chunk_scan_states_fwd(C, out, dA_cumsum, seq_idx, y, dims, accumulate, stream);
 }
 
 int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states, const ssd_tensor *dA_cumsum,

@@ -41,7 +41,13 @@ struct Params {
     int n_cu;             // compute units of the device (0: not known, the launchers then assume 256 in 8 XCDs)
     int ws_cleared;       // the launch in front of that kernel has cleared `ws` already (chain_workspace_clear below)
     int epoch;            // of this launch on `ws` (below); <= 0: contents unknown, the launcher clears it and takes 1
-    float *carry;         // inside `ws`, behind the flags: the fp32 states that cross between items when `out` is 16-bit
+    float *carry;         // inside `ws`, behind the flags: the fp32 states that cross between items when `out` is 16-bit or absent
+    // the scan's state half inside the chain kernel (null y: not wanted)
+    const void *Cm;       // (b, L, G, N), the element type of x
+    void *y;              // (b, L, H, P)
+    int64_t sC_b, sC_l, sC_g;
+    int64_t sy_b, sy_l, sy_h;
+    int dt_y, y_accumulate;
 };
 
 // State passing on a flattened state axis.
@@ -168,6 +174,9 @@ int set_quad_segment_chunks(int n);     // 0 = automatic; chunks per workgroup o
 // fused, work items drawn by ticket and chained by flags: every compute unit busy whatever the number of tiles
 hipError_t launch_chain(const Params &p, int n_cu, int mode, hipStream_t s);
 bool chain_supported(const Params &p);
+bool chain_needs_carry(const Params &p);      // the workspace also holds the fp32 states that cross between items
+// the variant of the chain kernel that also computes the scan's state half (p.y); the launch plan is launch_chain's
+hipError_t launch_chain_scan(const Params &p, int chunks_per_item, bool local, int n_wg, hipStream_t s);
 size_t chain_workspace_bytes(int batch, int nheads, int headdim, int nchunks);
 // ... and with room for the fp32 states that cross between items of `chunks_per_item` chunks when `out` is bf16
 size_t chain_workspace_bytes_out16(int batch, int nheads, int headdim, int dstate, int nchunks, int chunks_per_item);

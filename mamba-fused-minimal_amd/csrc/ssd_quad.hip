@@ -407,9 +407,13 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
     }
     put_weights(c0, 0, mcur);
     Frag fA, fB;
-    // B operands (transposed blocks) travel kAhead iterations ahead of the MFMAs that use them, across step
-    // boundaries: block t of the stream of (step, tile) pairs sits in slot t % 4.  An LDS read takes longer than the
-    // four MFMAs of one iteration, so a single block in flight would leave the matrix pipe waiting every iteration.
+    // B operands (transposed blocks) travel kAhead iterations ahead of the MFMAs that use them, across the step
+    // boundaries of a chunk: block t of the stream of (step, tile) pairs sits in slot t % 4.  An LDS read takes longer
+    // than the four MFMAs of one iteration, so a single block in flight would leave the matrix pipe waiting every
+    // iteration.  These are asynchronous results of inline assembly, which the compiler takes for complete: a value it
+    // has to carry around the chunk loop, or past its end, it may copy or overwrite before the data is there.  So none
+    // is in flight at the end of a chunk: the first blocks of a chunk are read at its top (the build checks the
+    // generated code for such copies, isa_check.py).
     constexpr int kAhead = 3;
     static_assert(NT % 4 == 0 && kAhead < 4 && kAhead <= NT, "slot of a block = its tile index % 4");
     // vector-memory operations of one store_state, at least (a 16-bit `out` takes NT stores, a 32-bit one 2 NT; the
@@ -430,11 +434,6 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         read_operands(0, 0, xr, wv);
 #pragma unroll
         for (int q = 0; q < 4; ++q) { frag_piece(q, 0, xr, wv, fA); frag_piece(q, 1, xr, wv, fA); }
-        __builtin_amdgcn_sched_barrier(0);
-        static_for<kAhead>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            read_Bt(std::integral_constant<int, 0>{}, ic, blo[i], bhi[i]);
-        });
         __builtin_amdgcn_sched_barrier(0);
     }
     int32_t prev_id = 0;
@@ -513,8 +512,9 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
             }
             {
                 constexpr int tn = it + kAhead;     // block kAhead iterations on: this step's tile or the next one's
-                read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
-                        blo[tn % 4], bhi[tn % 4]);
+                if constexpr (tn < NT || s + 1 < SPC)       // (the next chunk's first blocks: at its top)
+                    read_Bt(std::integral_constant<int, (tn < NT ? s : s + 1) % kRing>{}, std::integral_constant<int, tn % NT>{},
+                            blo[tn % 4], bhi[tn % 4]);
             }
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, h1, acc[it][1], 0, 0, 0);
@@ -533,6 +533,13 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
 
     for (int c = c0; c < C; ++c) {
         const int ws = (c - c0) & 1;
+        // the first blocks of step 0, whose tile every wave has published (prologue, or the barrier of the last step)
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<kAhead>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            read_Bt(std::integral_constant<int, 0>{}, ic, blo[i], bhi[i]);
+        });
+        __builtin_amdgcn_sched_barrier(0);
         step(c, std::integral_constant<int, 0>{}, ws, fA, fB);
         step(c, std::integral_constant<int, 1>{}, ws, fB, fA);
         step(c, std::integral_constant<int, 2>{}, ws, fA, fB);

@@ -476,6 +476,73 @@ def _chunk_scan_states_fwd(C, prev_states, dA_cumsum, seq_idx=None, out=None, ou
     return out
 
 
+def _fused_chunk_state_state_passing_scan_fwd(B, x, C, dt, dA_cumsum, out_dtype=torch.float32, initial_states=None,
+                                              seq_idx=None, y=None, y_dtype=None, accumulate=False, return_states=True,
+                                              _clamp=True, _kernel=0, _chunks_per_item=0, _workspace=None, _epoch=0,
+                                              _spin_limit=0):
+    """Chunk state + state passing + the state-dependent half of the chunk scan in one call
+    (ssd_fused_chunk_state_passing_scan_fwd): what the reference does with kernels/fused_concurrent.py:255-331 followed
+    by the state half of kernels/ssd_chunk_scan.py:94-117 (main.py:100-101).  Returns (out or None, final_states, y).
+
+    ``return_states=False`` leaves ``out`` -- (b,C,H,P,N), the state entering every chunk -- out altogether: where the
+    ticket / flag-chain kernel serves the call the passed states then never reach memory.  ``y`` (b,L,H,P) is created in
+    ``y_dtype`` (default C's, as the reference's scan output takes x's) unless given; ``accumulate=True`` adds to a given
+    ``y`` (the intra-chunk half of the scan computed elsewhere).  The other arguments are those of
+    ``_fused_chunk_state_state_passing_fwd``."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate) and C.shape == B.shape
+    assert dt.shape == (batch, nheads, nchunks, chunk_size) and dA_cumsum.shape == dt.shape
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+    _lib.require_device(x, "_fused_chunk_state_state_passing_scan_fwd")
+    lib = _lib.load()
+    if y is None:
+        assert not accumulate, "accumulate=True needs the tensor to add to (y=)"
+        y = torch.empty(batch, seqlen, nheads, headdim, device=x.device, dtype=y_dtype or C.dtype)
+    else:
+        assert y.shape == (batch, seqlen, nheads, headdim) and y.stride(-1) == 1
+    B, x, dt, dA_cumsum, seq_idx = _prep_inputs(B, x, dt, dA_cumsum, seq_idx)
+    if C.stride(-1) != 1:
+        C = C.contiguous()
+    if initial_states is not None and initial_states.stride(-1) != 1:
+        initial_states = initial_states.contiguous()
+    final_states = torch.empty((batch, nheads, headdim, dstate), device=x.device, dtype=torch.float32)
+    dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
+    T = _lib.tensor_arg
+    pairs = batch * nheads * ((headdim + 31) // 32) * nchunks
+    used = ctypes.c_int32(0)
+
+    def call(out):
+        def launch(workspace, epoch):
+            opts = _lib.SsdFusedOpts(workspace.data_ptr(), workspace.numel() * 4, int(_spin_limit), int(_kernel),
+                                     int(_chunks_per_item), int(epoch), ctypes.pointer(used))
+            with torch.cuda.device(x.device):
+                return lib.ssd_fused_chunk_state_passing_scan_fwd(
+                    T(x), T(B), T(C), T(dt), T(dA_cumsum), T(seq_idx), T(initial_states), T(out), T(final_states), T(y),
+                    dims, 1 if _clamp else 0, int(bool(accumulate)), ctypes.byref(opts), _stream(x))
+
+        if _workspace is not None:
+            return launch(_workspace, _epoch)
+        nbytes = int(lib.ssd_fused_scan_workspace_bytes(dims, 1 if out is not None else 0, int(_chunks_per_item)))
+        return _launch_on_own_workspace(x, nbytes, launch, used, pairs)
+
+    out = None
+    if return_states:
+        out = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=out_dtype or torch.float32)
+    rc = call(out)
+    if rc == _lib.SSD_ERR_SCRATCH and out is None and _kernel == 0:
+        # arguments the one-launch kernel does not take: the passed states then need a place, which this wrapper (the
+        # owner of all allocations) provides and drops again
+        rc = call(torch.empty((batch, nchunks, nheads, headdim, dstate), device=x.device, dtype=torch.float32))
+    _lib.check(rc, "ssd_fused_chunk_state_passing_scan_fwd")
+    return out, final_states, y
+
+
 def set_scan_kernel(kernel):
     """Tuning / test hook (no counterpart in the reference): 1 = the scan consumer runs one workgroup per head, 2 = one
     workgroup per run of heads wherever that kernel applies, 0 = let the library choose.  Returns the previous setting."""
