@@ -225,7 +225,38 @@ def main():
     # ... and on bf16 passed states (the reference's main.py hands its scan `out` in C's type)
     prev_states = [fused_bf16(i)[0] for i in range(nsets)]
     _, scan16_ev = timed(scan_states, steps_2nd, 3)
-    del prev_states, y_bufs
+    del prev_states
+    # path + consumer in one launch (ssd_fused_chunk_state_passing_scan_fwd): with the passed states as an output and
+    # fp32 y -- what the two calls above compute together --, and without them (bf16 y, the type the reference's scan
+    # writes; fp32 y), where they never reach memory
+    fscan = {}
+    if cfg["dtype"] == "bf16" and not args.with_states:
+        y16 = [torch.empty(b, L, H, P, device=dev, dtype=torch.bfloat16) for _ in range(nsets)]
+
+        def make(ret, ybufs):
+            def f(i):
+                s = sets[i % nsets]
+                return ssd_amd._fused_chunk_state_state_passing_scan_fwd(
+                    s["B"], s["x"], C_dev[i % nsets], s["dt"], s["dA_cumsum"], torch.float32, initial_states=s["initial_states"],
+                    seq_idx=s["seq_idx"], y=ybufs[i % nsets], return_states=ret)
+            return f
+
+        for key, ret, ybufs in (("fused_with_scan_states_us", True, y_bufs), ("fused_scan_without_passed_states_us", False, y_bufs),
+                                ("fused_scan_without_passed_states_bf16_y_us", False, y16)):
+            _, ev = timed(make(ret, ybufs), steps_2nd, 3)
+            assert ssd_amd.fused_status() == 0
+            fscan[key] = round(ev * 1e6, 2)
+        # parity of the last variant against the oracle on one batch row
+        o_, f_, y_ = make(False, y16)(0)
+        torch.cuda.synchronize()
+        wo, wf = ssd_oracle.fused_ref(d["B"][:1], d["x"][:1], d["dt"][:1], d["dA_cumsum"][:1],
+                                      initial_states=None if d["initial_states"] is None else d["initial_states"][:1],
+                                      seq_idx=None if d["seq_idx"] is None else d["seq_idx"][:1])
+        wy = ssd_oracle.chunk_scan_states_ref(d["C"][:1], wo, d["dA_cumsum"][:1], seq_idx=None if d["seq_idx"] is None else d["seq_idx"][:1])
+        ey = (y_[:1].float().cpu() - wy).abs()
+        fscan["fused_scan_parity_mismatches"] = int((ey > 1e-3 + (2e-3 + 2.0 ** -8) * wy.abs()).sum())
+        del y16, o_, f_, y_
+    del y_bufs
     # the headline call again without the clock ramp, right after host-side idling: what a lone call in a quiet stream sees
     torch.cuda.synchronize()
     time.sleep(0.5)
@@ -297,6 +328,7 @@ def main():
         "fused_with_dt_preparation_us": round(prep_ev * 1e6, 2),
         "chunk_scan_states_us": round(scan_ev * 1e6, 2),
         "chunk_scan_states_from_bf16_us": round(scan16_ev * 1e6, 2),
+        **fscan,
         "fused_speedup_vs_unfused": round(unf_ev / ev_step, 3),
         "parity_mismatches": bad,
         "parity_scope": scope,

@@ -345,8 +345,8 @@ int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states
  * what y holds.  `out` MAY BE ABSENT (out == NULL or out->data == NULL): then the only trace of the passed states is
  * one 32 x dstate fp32 slot per (state tile, work item) in the workspace, and final_states.  opts: as in
  * ssd_fused_chunk_state_passing_fwd_ws; the workspace must hold ssd_fused_scan_workspace_bytes(dims, with_out,
- * opts->chunks_per_item) bytes, 16-byte aligned (with_out: `out` is given, fp32; work items are two chunks long with
- * dstate 128 -- what the register file holds next to the operands of the second product -- and up to four with dstate 64).
+ * opts->chunks_per_item) bytes, 16-byte aligned (with_out: `out` is given, fp32; work items are two chunks long
+ * whatever chunks_per_item says -- what the register file holds next to the operands of the second product).
  * The one-launch kernel takes what the chain kernel takes (bf16 x / B / C, fp32 out if any, dstate 64 or 128, chunk 128
  * or 256, four state tiles per (batch, group), 16-byte aligned rows) and needs the workspace.  Any other call WITH `out`
  * runs as ssd_fused_chunk_state_passing_fwd[_ws] followed by ssd_chunk_scan_states_fwd (*opts->used_workspace says which

@@ -17,8 +17,6 @@ FLAGS = [
     # keep the compiler from forming packed-fp32 VALU instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
-    # one remark block per kernel with its registers, spills and scratch: collected into build/resource_usage.json
-    "-Rpass-analysis=kernel-resource-usage",
 ]
 USAGE = os.path.join(OBJ_DIR, "resource_usage.json")
 ISA_CHECK = os.path.join(OBJ_DIR, "async_operand_check.json")
@@ -40,26 +38,24 @@ def _run(cmd):
     return out
 
 
-def _resource_usage(text):
-    """Splits a compiler log into ({kernel: {field: value}}, the log without the resource-usage remarks)."""
+def _resource_usage(asm_text):
+    """{kernel: {field: value}} from the gfx950 assembly the compiler leaves behind (--save-temps): the metadata entry of
+    every kernel (registers, spills, scratch, dynamic stack) and the occupancy the compiler notes beside its code."""
     import re
-    usage, rest, current, skip = {}, [], None, 0
-    for line in text.splitlines():
-        m = re.search(r"remark:\s+(.*?)\s+\[-Rpass-analysis=kernel-resource-usage\]", line)
-        if m:
-            key, _, value = m.group(1).partition(": ")
-            if key == "Function Name":
-                current = usage.setdefault(value.strip(), {})
-            elif current is not None:
-                value = value.strip()
-                current[key.strip()] = int(value) if value.lstrip("-").isdigit() else value
-            skip = 2                      # the source line and the caret that follow a remark
-        elif skip and (line.lstrip().startswith("|") or re.match(r"\s*\d+ \|", line)):
-            skip -= 1
-        else:
-            skip = 0
-            rest.append(line)
-    return usage, "\n".join(rest)
+    usage = {}
+    occupancy = {}
+    for m in re.finditer(r"^\s*\.amdhsa_kernel (\S+)$(.*?)^; Occupancy: (\d+)", asm_text, re.M | re.S):
+        occupancy[m.group(1)] = int(m.group(3))
+    for entry in re.split(r"^  - ", asm_text[asm_text.rfind("amdhsa.kernels:"):], flags=re.M)[1:]:
+        f = dict(re.findall(r"^\s*\.(\w+):\s+(\S+)\s*$", entry, re.M))
+        if "name" not in f:
+            continue
+        agpr, total = int(f.get("agpr_count", 0)), int(f.get("vgpr_count", 0))
+        usage[f["name"]] = {"VGPRs": total - agpr, "AGPRs": agpr, "ScratchSize [bytes/lane]": int(f.get("private_segment_fixed_size", 0)),
+                            "VGPRs Spill": int(f.get("vgpr_spill_count", 0)), "SGPRs Spill": int(f.get("sgpr_spill_count", 0)),
+                            "Dynamic Stack": "True" if f.get("uses_dynamic_stack") == "true" else "False",
+                            "Occupancy [waves/SIMD]": occupancy.get(f["name"], 0)}
+    return usage
 
 
 def build_library(verbose=False, extra_flags=(), jobs=None):
@@ -91,14 +87,20 @@ def build_library(verbose=False, extra_flags=(), jobs=None):
     # the generated code, checked for copies of operands that inline assembly is still loading (isa_check.py)
     sys.path.insert(0, HERE)
     import isa_check
-    findings = {}
+    findings, usage = {}, {}
     for src in SOURCES:
         tmp = os.path.join(OBJ_DIR, "temps_" + os.path.splitext(src)[0])
+        usage[src] = {}
         for name in sorted(os.listdir(tmp)):
             if name.endswith("gfx950.s"):
-                findings[src] = isa_check.check_file(os.path.join(tmp, name))
+                with open(os.path.join(tmp, name)) as f:
+                    text = f.read()
+                findings[src] = isa_check.check_text(text)
+                usage[src] = _resource_usage(text)
         shutil.rmtree(tmp, ignore_errors=True)
     import json
+    with open(USAGE, "w") as f:
+        json.dump(usage, f, indent=1, sort_keys=True)
     with open(ISA_CHECK, "w") as f:
         json.dump(findings, f, indent=1, sort_keys=True)
     bad = {k: v for k, v in findings.items() if v}
@@ -107,13 +109,9 @@ def build_library(verbose=False, extra_flags=(), jobs=None):
         raise RuntimeError(f"the compiler moved operands that inline assembly is still loading in {sorted(bad)} "
                            f"({sum(len(v) for v in bad.values())} places, e.g. {first}); see {ISA_CHECK}")
     out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in results], "-o", LIB])
-    usage = {}
     for src, (_, text) in zip(SOURCES, results):
-        usage[src], rest = _resource_usage(text)
-        if verbose and rest.strip():
-            print(rest)
-    with open(USAGE, "w") as f:
-        json.dump(usage, f, indent=1, sort_keys=True)
+        if verbose and text.strip():
+            print(text)
     if verbose and out.strip():
         print(out)
     return LIB

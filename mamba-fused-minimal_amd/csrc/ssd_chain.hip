@@ -77,15 +77,12 @@ size_t chain_workspace_bytes_out16(int batch, int nheads, int headdim, int dstat
 // of the passed states would be a whole fp32 `out`.
 int chain_chunks_per_item(const Params &p, int n_cu, int forced)
 {
-    if (p.y && (forced == 1 || (forced == 4 && p.dstate > 64))) forced = 2;
+    if (p.y) return 2;        // the variant that also computes the scan's state half: what the register file holds
     if (forced == 1 || forced == 2 || forced == 4) return forced;
     cost::Problem q;
     q.units = (p.batch * p.nheads * (p.headdim / 32)) >> 2; q.chunks = p.C; q.chunk_size = p.Q; q.dstate = p.dstate;
     q.n_cu = n_cu > 0 ? n_cu : 256;
     const int r = cost::chain_chunks_per_item(q, nullptr);
-    // the variant that also computes the scan's state half exists for items of two chunks, and of four with dstate 64
-    // (what the register file holds)
-    if (p.y) return p.dstate > 64 || r < 4 ? 2 : 4;
     return chain_needs_carry(p) && r < 2 ? 2 : r;
 }
 
@@ -179,7 +176,6 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     // Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units
     // end up with too few or too unequal numbers of items that large.  p.n_seg > 0 forces a value.
     const int r = chain_chunks_per_item(p, n_cu, p.n_seg);
-    if (p.y && r < 2) return hipErrorInvalidValue;
     if (chain_needs_carry(p)) {
         if (r < 2) return hipErrorInvalidValue;
         p.carry = (float *)(p.ws + carry_offset_ints(p.n_items, p.C));

@@ -470,26 +470,32 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         // tile t of the item = step t % SPC of chunk c0 + t / SPC; a wave fetches NTW of its NT blocks (16 tokens x 32
         // columns, 1 KB: lane l the 16 bytes (token l/4, piece (l%4) ^ (l/16)), so that the operand reads of 16 tokens
         // at one piece fall on 16 different bank groups); tiles past the item's end: requests that fetch nothing
-        auto load_C = [&](int t) {
+        // The request cursor: the next tile to ask for, its chunk's descriptor pieces and its ring slot.
+        int rq_t = 0, rq_st = 0, rq_slot = 0;
+        const char *rq_base = I.Cb + (int64_t)c0 * Q * Crb;       // first row of the chunk
+        int64_t rq_bytes = (int64_t)(L - c0 * Q) * Crb;           // rows of the sequence from there on
+        auto load_C = [&]() {
 #if defined(__HIP_DEVICE_COMPILE__)
             typedef __attribute__((address_space(3))) void *lds_ptr;
-            const int j = t / SPC, st = t - j * SPC, c = c0 + j;
-            const __amdgpu_buffer_rsrc_t rs = make_rsrc(I.Cb + (int64_t)c * Q * Crb, t < n_tiles ? (int64_t)(L - c * Q) * Crb : 0);
-            char *dst = cring + (t % kRingC) * NT * 1024;
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(rq_base, rq_t < n_tiles ? rq_bytes : 0);
+            char *dst = cring + rq_slot * NT * 1024;
 #pragma unroll
             for (int k = 0; k < NTW; ++k) {
                 const int bi = wave * NTW + k, th = bi / (NT / 2), pair = bi % (NT / 2);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(dst + bi * 1024), 16, Clane, (int)((32 * st + 16 * th) * Crb) + 64 * pair, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(dst + bi * 1024), 16, Clane, (int)((32 * rq_st + 16 * th) * Crb) + 64 * pair, 0, 0);
             }
+            ++rq_t;
+            rq_slot = rq_slot + 1 == kRingC ? 0 : rq_slot + 1;
+            if (++rq_st == SPC) { rq_st = 0; rq_base += (int64_t)Q * Crb; rq_bytes -= (int64_t)Q * Crb; }
 #else
-            (void)t; (void)Clane; (void)n_tiles;
+            (void)Clane; (void)n_tiles; (void)rq_t; (void)rq_st; (void)rq_slot; (void)rq_base; (void)rq_bytes;
 #endif
         };
         float ycs[R][TPL];
         int32_t yid[R][TPL], yprev[R];
         if constexpr (SCAN) {
 #pragma unroll 1
-            for (int t = 0; t < kDistC; ++t) load_C(t);
+            for (int t = 0; t < kDistC; ++t) load_C();
             static_for<R>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 if (j < n) {
@@ -616,10 +622,98 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            int t = 0;
-#if defined(SSD_SCAN_DBG) && SSD_SCAN_DBG == 1
-            if (p.batch > 0) return;
-#endif
+            int slot = 0;                                        // ring slot of the tile consumed next
+            // C operands (lane (token i16, kg): columns 32u + 4kg .. + 3 and 32u + 16 + 4kg .. + 3 of slab u) and per-token
+            // scales of the two 16-token blocks of a tile
+            struct TileOps { bf16x8 cop[2][NT / 2]; float sc[2]; };
+            // A tile has landed once no more operations are outstanding than were issued behind its requests (those of
+            // the kDistC - 1 tiles after it and the loads and stores of kDistC tiles); the barrier publishes every
+            // wave's blocks and says that all waves are through with the tile before, whose slot the next request
+            // overwrites.  Then the tile's operands are read.
+            auto open_tile = [&](int st, TileOps &o) {
+                constexpr int kReq = (kDistC - 1) * NTW;
+                if (mode == 0) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 2));
+                else if (mode == 1 || mode == 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 4));
+                else __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 8));
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                load_C();
+                const char *tile_c = cring + slot * NT * 1024;
+                slot = slot + 1 == kRingC ? 0 : slot + 1;
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+                    for (int u = 0; u < NT / 2; ++u) {
+                        const char *blk = tile_c + (tb * (NT / 2) + u) * 1024 + 64 * i16 + 8 * (kg & 1);
+                        const u32x2 c0v = *(const u32x2 *)(blk + 16 * ((kg >> 1) ^ (i16 >> 2)));
+                        const u32x2 c1v = *(const u32x2 *)(blk + 16 * ((2 + (kg >> 1)) ^ (i16 >> 2)));
+                        o.cop[tb][u] = __builtin_bit_cast(bf16x8, (u32x4){c0v.x, c0v.y, c1v.x, c1v.y});
+                    }
+                    o.sc[tb] = *(const float *)(wbuf + ws_free * Q * 4 + 4 * (32 * st + 16 * tb + i16));
+                }
+            };
+            // the tile's two blocks: 2 x NT matrix instructions each, then the results scaled, turned into rows through
+            // LDS and stored
+            auto finish_tile = [&](int st, const TileOps &o, __amdgpu_buffer_rsrc_t rsy) {
+                f32x4 Dv[2][2];
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    f32x4 D0 = {0.f, 0.f, 0.f, 0.f}, D1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int u = 0; u < NT / 2; ++u) {
+                        D0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[0][u]), o.cop[tb][u], D0, 0, 0, 0);
+                        D1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[1][u]), o.cop[tb][u], D1, 0, 0, 0);
+                        D0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[0][u]), o.cop[tb][u], D0, 0, 0, 0);
+                        D1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[1][u]), o.cop[tb][u], D1, 0, 0, 0);
+                    }
+                    Dv[tb][0] = D0; Dv[tb][1] = D1;
+                }
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    const f32x4 D0 = Dv[tb][0], D1 = Dv[tb][1];
+                    // lane (token i16, kg): D0[r] / D1[r] = headdim rows p0 + 8kg + 2r / + 2r + 1 -- eight consecutive
+                    // values of the token's y row; through LDS they become (lane/4 = token, lane%4 = piece), so that
+                    // four adjacent lanes address 64 (fp32: 2 x 64) contiguous bytes
+                    const float sc = o.sc[tb];
+                    const float v[8] = {D0.x * sc, D1.x * sc, D0.y * sc, D1.y * sc, D0.z * sc, D1.z * sc, D0.w * sc, D1.w * sc};
+                    char *wr = stage + i16 * 64 + ((kg ^ (i16 >> 2)) << 4);
+                    const char *rd = stage + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4);
+                    const int tok = 32 * st + 16 * tb;           // first token of the block
+                    if (mode == 0) {
+                        *(u32x4 *)wr = (u32x4){pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+                        const u32x4 q = *(const u32x4 *)rd;
+                        __builtin_amdgcn_raw_buffer_store_b128(q, rsy, (int)((lane >> 2) * yrb) + 16 * (lane & 3), (int)(tok * yrb), 0);
+                        asm volatile("s_nop 3" ::"v"(q) : "memory");
+                    } else {
+                        // fp32 in flight: two passes of four values each
+                        *(f32x4 *)wr = (f32x4){v[0], v[1], v[2], v[3]};
+                        f32x4 a = *(const f32x4 *)rd;
+                        *(f32x4 *)wr = (f32x4){v[4], v[5], v[6], v[7]};
+                        f32x4 d = *(const f32x4 *)rd;
+                        if (p.dt_y == DT_F32) {
+                            const int voff = (int)((lane >> 2) * yrb) + 32 * (lane & 3);
+                            if (p.y_accumulate) {
+                                a += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb), 0));
+                                d += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb) + 16, 0));
+                            }
+                            const u32x4 qa = __builtin_bit_cast(u32x4, a), qd = __builtin_bit_cast(u32x4, d);
+                            __builtin_amdgcn_raw_buffer_store_b128(qa, rsy, voff, (int)(tok * yrb), 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(qd, rsy, voff, (int)(tok * yrb) + 16, 0);
+                            asm volatile("s_nop 3" ::"v"(qa), "v"(qd) : "memory");
+                        } else {
+                            const int voff = (int)((lane >> 2) * yrb) + 16 * (lane & 3);
+                            const u32x4 o_ = __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb), 0);
+                            const float f[8] = {a.x, a.y, a.z, a.w, d.x, d.y, d.z, d.w};
+                            u32x4 q;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                q[e] = pack_bf16(f[2 * e] + bf16_bits_to_f32(o_[e] & 0xffffu), f[2 * e + 1] + bf16_bits_to_f32(o_[e] >> 16));
+                            __builtin_amdgcn_raw_buffer_store_b128(q, rsy, voff, (int)(tok * yrb), 0);
+                            asm volatile("s_nop 3" ::"v"(q) : "memory");
+                        }
+                    }
+                }
+            };
 #pragma unroll 1
             for (int j = 0; j < n; ++j) {
                 static_for<R>([&](auto jc) {
@@ -641,79 +735,17 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
                 const int c = c0 + j;
                 const int rows = min(Q, L - c * Q);
                 const __amdgpu_buffer_rsrc_t rsy = make_rsrc(yb + (int64_t)c * Q * yrb, (int64_t)(rows - 1) * yrb + 32 * esz);
+                // Two tiles per trip: the operands of a tile are read in front of the matrix instructions of the tile
+                // before it, so that their way from LDS (and the wait and the barrier in front of it) runs beside those
+                // instructions.  A chunk's first tile has nothing in front of it: the conversion above.
+                TileOps oa, ob;
+                open_tile(0, oa);
 #pragma unroll 1
-                for (int st = 0; st < SPC; ++st, ++t) {
-                    // tile t has landed once no more operations are outstanding than were issued behind its requests
-                    // (those of the kDistC - 1 tiles after it and the loads and stores of kDistC tiles); the barrier
-                    // publishes every wave's blocks and says that all are through with tile t - 1, whose slot the
-                    // requests below overwrite
-                    constexpr int kReq = (kDistC - 1) * NTW;
-                    if (mode == 0) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 2));
-                    else if (mode == 1 || mode == 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 4));
-                    else __builtin_amdgcn_s_waitcnt(vmcnt_imm(kReq + kDistC * 8));
-                    __builtin_amdgcn_s_barrier();
-                    asm volatile("" ::: "memory");
-                    load_C(t + kDistC);
-                    const char *tile_c = cring + (t % kRingC) * NT * 1024;
-#pragma unroll
-                    for (int tb = 0; tb < 2; ++tb) {
-                        f32x4 D0 = {0.f, 0.f, 0.f, 0.f}, D1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int u = 0; u < NT / 2; ++u) {
-                            const char *blk = tile_c + (tb * (NT / 2) + u) * 1024 + 64 * i16 + 8 * (kg & 1);
-                            const u32x2 c0v = *(const u32x2 *)(blk + 16 * ((kg >> 1) ^ (i16 >> 2)));
-                            const u32x2 c1v = *(const u32x2 *)(blk + 16 * ((2 + (kg >> 1)) ^ (i16 >> 2)));
-                            const bf16x8 cop = __builtin_bit_cast(bf16x8, (u32x4){c0v.x, c0v.y, c1v.x, c1v.y});
-                            D0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[0][u]), cop, D0, 0, 0, 0);
-                            D1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, shi[1][u]), cop, D1, 0, 0, 0);
-                            D0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[0][u]), cop, D0, 0, 0, 0);
-                            D1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, slo[1][u]), cop, D1, 0, 0, 0);
-                        }
-                        // lane (token i16, kg): D0[r] / D1[r] = headdim rows p0 + 8kg + 2r / + 2r + 1 -- eight consecutive
-                        // values of the token's y row; through LDS they become (lane/4 = token, lane%4 = piece), so that
-                        // four adjacent lanes address 64 (fp32: 2 x 64) contiguous bytes
-                        const float sc = *(const float *)(wbuf + ws_free * Q * 4 + 4 * (32 * st + 16 * tb + i16));
-                        const float v[8] = {D0.x * sc, D1.x * sc, D0.y * sc, D1.y * sc, D0.z * sc, D1.z * sc, D0.w * sc, D1.w * sc};
-                        char *wr = stage + i16 * 64 + ((kg ^ (i16 >> 2)) << 4);
-                        const char *rd = stage + (lane >> 2) * 64 + (((lane & 3) ^ (lane >> 4)) << 4);
-                        const int tok = 32 * st + 16 * tb;           // first token of the block
-#if defined(SSD_SCAN_DBG) && SSD_SCAN_DBG == 2
-                        if (p.batch > 0) { if (v[0] == 1.2345f) *(float *)wr = 0.f; continue; }
-#endif
-                        if (mode == 0) {
-                            *(u32x4 *)wr = (u32x4){pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
-                            const u32x4 q = *(const u32x4 *)rd;
-                            __builtin_amdgcn_raw_buffer_store_b128(q, rsy, (int)((lane >> 2) * yrb) + 16 * (lane & 3), (int)(tok * yrb), 0);
-                            asm volatile("s_nop 3" ::"v"(q) : "memory");
-                        } else {
-                            // fp32 in flight: two passes of four values each
-                            *(f32x4 *)wr = (f32x4){v[0], v[1], v[2], v[3]};
-                            f32x4 a = *(const f32x4 *)rd;
-                            *(f32x4 *)wr = (f32x4){v[4], v[5], v[6], v[7]};
-                            f32x4 d = *(const f32x4 *)rd;
-                            if (p.dt_y == DT_F32) {
-                                const int voff = (int)((lane >> 2) * yrb) + 32 * (lane & 3);
-                                if (p.y_accumulate) {
-                                    a += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb), 0));
-                                    d += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb) + 16, 0));
-                                }
-                                const u32x4 qa = __builtin_bit_cast(u32x4, a), qd = __builtin_bit_cast(u32x4, d);
-                                __builtin_amdgcn_raw_buffer_store_b128(qa, rsy, voff, (int)(tok * yrb), 0);
-                                __builtin_amdgcn_raw_buffer_store_b128(qd, rsy, voff, (int)(tok * yrb) + 16, 0);
-                                asm volatile("s_nop 3" ::"v"(qa), "v"(qd) : "memory");
-                            } else {
-                                const int voff = (int)((lane >> 2) * yrb) + 16 * (lane & 3);
-                                const u32x4 o = __builtin_amdgcn_raw_buffer_load_b128(rsy, voff, (int)(tok * yrb), 0);
-                                const float f[8] = {a.x, a.y, a.z, a.w, d.x, d.y, d.z, d.w};
-                                u32x4 q;
-#pragma unroll
-                                for (int e = 0; e < 4; ++e)
-                                    q[e] = pack_bf16(f[2 * e] + bf16_bits_to_f32(o[e] & 0xffffu), f[2 * e + 1] + bf16_bits_to_f32(o[e] >> 16));
-                                __builtin_amdgcn_raw_buffer_store_b128(q, rsy, voff, (int)(tok * yrb), 0);
-                                asm volatile("s_nop 3" ::"v"(q) : "memory");
-                            }
-                        }
-                    }
+                for (int st = 0; st < SPC; st += 2) {
+                    open_tile(st + 1, ob);
+                    finish_tile(st, oa, rsy);
+                    if (st + 2 < SPC) open_tile(st + 2, oa);
+                    finish_tile(st + 1, ob, rsy);
                 }
             }
         }

@@ -34,11 +34,14 @@ def test_every_source_reports_its_kernels(usage):
     counts = {src: len(kernels) for src, kernels in usage.items()}
     assert counts["ssd_capi.hip"] == 0                       # host code only
     for src in ("ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_generic.hip", "ssd_state_passing.hip",
-                "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip"):
+                "ssd_chunk_cumsum.hip", "ssd_chunk_scan_states.hip", "ssd_mover.hip", "ssd_chain_scan.hip"):
         assert counts[src] > 0, src
     # the chain kernel: dstate 64 / 128 x chunk 128 / 256 x 1 / 2 / 4 chunks per item (2 / 4 with bf16 out) x seq_idx or
     # not x LOCAL / GLOBAL, + the fill
     assert counts["ssd_chain.hip"] == 4 * (3 + 2) * 2 * 2 + 1
+    # ... and with the scan's state half in its chain step (items of two chunks): out fp32 or absent x seq_idx x
+    # LOCAL / GLOBAL x chunk 128 / 256 x dstate 64 / 128
+    assert counts["ssd_chain_scan.hip"] == 2 * 2 * 2 * 2 * 2
 
 
 def test_no_kernel_spills_vector_registers_or_uses_scratch(usage):
@@ -57,3 +60,38 @@ def test_register_budgets_of_the_two_four_tile_kernels(usage):
         assert r["VGPRs"] + r["AGPRs"] <= 256 and r["Occupancy [waves/SIMD]"] >= 2, (name, r)
     big = [r for name, r in usage["ssd_chain.hip"].items() if "chain_kernelILi8ELi8ELi4E" in name]
     assert len(big) == 8 and all(448 < r["VGPRs"] + r["AGPRs"] <= 512 for r in big), big
+
+
+def test_generated_code_has_no_copies_of_operands_in_flight(usage):
+    """The step loops read B operands with inline assembly whose results arrive later (an explicit wait in a later
+    statement); a compiler copy of such a result, or a reuse of its registers, in between gives silently wrong states.
+    The build scans the gfx950 assembly of every kernel for it (isa_check.py) and refuses to produce a library
+    otherwise; the record of the last build must be clean, for every source file."""
+    with open(os.path.join(PKG, "build", "async_operand_check.json")) as f:
+        findings = json.load(f)
+    assert set(findings) == set(usage)
+    assert all(v == [] for v in findings.values()), {k: v[:2] for k, v in findings.items() if v}
+
+
+def test_the_check_of_the_generated_code_finds_what_it_is_for():
+    import sys
+    sys.path.insert(0, PKG)
+    import isa_check
+    clean = """
+_Z6kernelv:
+	ds_read_b64_tr_b16 v[10:11], v5 offset:0
+	ds_read_b64_tr_b16 v[12:13], v5 offset:0x100
+	v_add_u32_e32 v1, v2, v3
+	s_waitcnt lgkmcnt(0)
+	v_mfma_f32_16x16x32_bf16 a[0:3], v[10:13], v[20:23], a[0:3]
+	v_mov_b32_e32 v10, v1
+	s_endpgm
+"""
+    assert isa_check.check_text(clean) == []
+    copied = clean.replace("v_add_u32_e32 v1, v2, v3", "v_accvgpr_write_b32 a9, v11")
+    found = isa_check.check_text(copied)
+    assert len(found) == 1 and found[0]["registers"] == [11] and found[0]["kernel"] == "_Z6kernelv"
+    reused = clean.replace("v_add_u32_e32 v1, v2, v3", "v_add_u32_e32 v12, v2, v3")
+    assert [f["registers"] for f in isa_check.check_text(reused)] == [[12]]
+    never_used = clean.replace("\tv_mfma_f32_16x16x32_bf16 a[0:3], v[10:13], v[20:23], a[0:3]\n", "")
+    assert len(isa_check.check_text(never_used)) == 1          # overwritten by the v_mov without ever landing in a use
