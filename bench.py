@@ -40,7 +40,7 @@ MEASURED_TRAFFIC = {
     "cfg3_varlen_packed": {"bytes": 861720134, "sources": "9b04869304ef2b26"},
     "cfg4_long_grouped": {"bytes": 5345658293, "sources": "9b04869304ef2b26"},
 }
-KERNEL_SOURCES = ("ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_tile.h", "ssd_params.h", "ssd_capi.hip")
+KERNEL_SOURCES = ("ssd_chain_kernel.h", "ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_tile.h", "ssd_params.h", "ssd_capi.hip")
 
 
 def kernel_source_hash():

@@ -348,10 +348,30 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             dst[k] = *rd;
         }
     };
+    // The state entering an item, fetched early.  The last of an item's R parking places is free until its last chunk
+    // ends; where the predecessor's flag is already up when that chunk starts -- the rule once every compute unit
+    // has its rhythm: the predecessor finished most of an item ago --, the state is read into that place while the
+    // chunk's steps run (early_fetch, called from the steps) and enters the recurrence here, before the place is
+    // taken.  The chain step then neither polls nor waits for a read.  Not where the scan's state half needs that state
+    // once more, nor for single-chunk items.
+    constexpr bool EARLY = !SCAN && R > 1;
+    bool early_have = false;          // held[R - 1] holds the state entering the current item
+    int early_flag = 0;
     auto park = [&](const Item &I, const Meta &m) {
         float sc = __expf(m.last);
         if (HAS_SEQ && m.id_last != m.id_prev) sc = 0.f;
         sc = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, sc)));
+        if constexpr (EARLY) {
+            if (I.r == R - 1 && early_have) {
+                const float s0 = scale[0];
+#pragma unroll
+                for (int k = 0; k < 2 * NT; ++k) {
+                    const f32x4 pv = held[R - 1][k];
+                    held[0][k] = (f32x4){__builtin_fmaf(pv.x, s0, held[0][k].x), __builtin_fmaf(pv.y, s0, held[0][k].y),
+                                         __builtin_fmaf(pv.z, s0, held[0][k].z), __builtin_fmaf(pv.w, s0, held[0][k].w)};
+                }
+            }
+        }
         static_for<R>([&](auto rc) {
             constexpr int r = decltype(rc)::value;
             if (I.r == r) { park_into(held[r]); scale[r] = sc; }
@@ -365,6 +385,38 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         if (lane == 0) {
             if (LOCAL) *(volatile int *)f = epoch;
             else __hip_atomic_store(f, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+    // where the state entering the item that starts at chunk c0 > 0 of I's tile lies: out[:, c0], or the fp32 slot of
+    // the workspace (a slot holds the tile's 32 rows only)
+    constexpr int kCarrySlotBytes = 32 * NT * 16 * 4;
+    auto entering_state = [&](const Item &I, int c0, int &pitch, int &row0) {
+        pitch = CARRY ? NT * 16 : (int)p.so_p;
+        row0 = CARRY ? 0 : I.p0;
+        if (CARRY) return make_rsrc((const char *)p.carry + ((int64_t)I.tile * n_super + c0 / R) * kCarrySlotBytes, kCarrySlotBytes);
+        return make_rsrc((const float *)p.out + I.b * p.so_b + I.h * p.so_h + (int64_t)c0 * p.so_c,
+                         ((int64_t)(p.headdim - 1) * p.so_p + p.dstate) * 4);
+    };
+    // Steps 0 and 2 of an item's last chunk (I.r == R - 1: the item has all its R chunks, and scale[0] is known): look
+    // at the predecessor's flag, and two steps later -- the answer has arrived behind the requests of those steps --
+    // ask for the state if it is up.
+    auto early_fetch = [&](const Item &I, int s) {
+        if constexpr (EARLY) {
+            const int c0 = I.c - I.r;
+            const bool wanted = I.r == R - 1 && c0 > 0 && scale[0] != 0.f;
+            if (s == 0) {
+                early_have = false;
+                if (wanted) early_flag = load_flag(ws_flags + (int64_t)I.tile * C + c0);
+            } else if (wanted && __builtin_amdgcn_readfirstlane(early_flag) == epoch) {
+                int pitch, row0;
+                const __amdgpu_buffer_rsrc_t rs = entering_state(I, c0, pitch, row0);
+                const int row = row0 + 2 * (lane >> 2), col = 4 * (lane & 3);
+#pragma unroll
+                for (int k = 0; k < 2 * NT; ++k)
+                    held[R - 1][k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                                   rs, 4 * (row * pitch + col), 4 * ((k & 1) * pitch + 16 * (k >> 1)), kAux));
+                early_have = true;
+            }
         }
     };
     // I: the last chunk of the item (chunks I.c - I.r .. I.c)
@@ -526,7 +578,8 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             hand_on();
         }
 
-        if (SCAN ? c0 > 0 : (use_prev && c0 > 0)) {
+        const bool early = EARLY && early_have && n == R && c0 > 0;     // the entering state is in held[0] already
+        if (!early && (SCAN ? c0 > 0 : (use_prev && c0 > 0))) {
             // out[:, c0] of this tile is complete once its flag is up
             int polls = 0;
             while (load_flag(flag + c0) != epoch) {
@@ -539,7 +592,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             asm volatile("" ::: "memory");
         }
         f32x4 s[2 * NT];       // the state entering the item
-        if (use_prev || c0 == 0 || SCAN) {
+        if (!early && (use_prev || c0 == 0 || SCAN)) {
             // chunk 0 copies initial_states to out[:, 0] even if a sequence boundary wipes them out at once
             const bool read = use_prev || p.init != nullptr || (SCAN && c0 > 0);
 #pragma unroll
@@ -870,6 +923,7 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         else read_operands(0, ws ^ 1, xr, wv);
         if (s == 0 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
             t_new = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (s == 0 || s == 2) early_fetch(cur, s);
         // published by this step's barrier: the ticket after next, or (first item) the next one and then that
         if (s == SPC - 2 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
             tq[second_late && cur.r == 0 ? 1 : 2] = t_new;
