@@ -233,17 +233,21 @@ def main():
     if cfg["dtype"] == "bf16" and not args.with_states:
         y16 = [torch.empty(b, L, H, P, device=dev, dtype=torch.bfloat16) for _ in range(nsets)]
 
-        def make(ret, ybufs):
+        def make(ret, ybufs, kern=0):
             def f(i):
                 s = sets[i % nsets]
                 return ssd_amd._fused_chunk_state_state_passing_scan_fwd(
                     s["B"], s["x"], C_dev[i % nsets], s["dt"], s["dA_cumsum"], torch.float32, initial_states=s["initial_states"],
-                    seq_idx=s["seq_idx"], y=ybufs[i % nsets], return_states=ret)
+                    seq_idx=s["seq_idx"], y=ybufs[i % nsets], return_states=ret, _kernel=kern)
             return f
 
-        for key, ret, ybufs in (("fused_with_scan_states_us", True, y_bufs), ("fused_scan_without_passed_states_us", False, y_bufs),
-                                ("fused_scan_without_passed_states_bf16_y_us", False, y16)):
-            _, ev = timed(make(ret, ybufs), steps_2nd, 3)
+        # headline of the one-launch entry: no passed states in memory, y in the type the reference's scan writes
+        # (C's: bf16); then fp32 y; then with `out` as well, which the library runs as its two stand-alone calls
+        # unless the one-launch kernel is insisted on (last figure)
+        for key, ret, ybufs, kern in (("fused_with_scan_states_us", False, y16, 0), ("fused_with_scan_states_fp32_y_us", False, y_bufs, 0),
+                                      ("fused_with_scan_states_and_out_fp32_y_us", True, y_bufs, 0),
+                                      ("fused_with_scan_states_and_out_one_launch_us", True, y_bufs, 1)):
+            _, ev = timed(make(ret, ybufs, kern), steps_2nd, 3)
             assert ssd_amd.fused_status() == 0
             fscan[key] = round(ev * 1e6, 2)
         # parity of the last variant against the oracle on one batch row

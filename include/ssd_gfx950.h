@@ -348,10 +348,12 @@ int ssd_chunk_scan_states_fwd(const ssd_tensor *C, const ssd_tensor *prev_states
  * opts->chunks_per_item) bytes, 16-byte aligned (with_out: `out` is given, fp32; work items are two chunks long
  * whatever chunks_per_item says -- what the register file holds next to the operands of the second product).
  * The one-launch kernel takes what the chain kernel takes (bf16 x / B / C, fp32 out if any, dstate 64 or 128, chunk 128
- * or 256, four state tiles per (batch, group), 16-byte aligned rows) and needs the workspace.  Any other call WITH `out`
- * runs as ssd_fused_chunk_state_passing_fwd[_ws] followed by ssd_chunk_scan_states_fwd (*opts->used_workspace says which
- * happened); without `out` and without that kernel there is no place for the passed states: SSD_ERR_SCRATCH (the
- * library never allocates).
+ * or 256, four state tiles per (batch, group), 16-byte aligned rows) and needs the workspace; with SSD_KERNEL_AUTO it
+ * serves the calls WITHOUT `out` -- with `out` it saves no traffic and is slower than the two calls, so it runs there
+ * only where opts->kernel insists.  Any other call WITH `out` runs as ssd_fused_chunk_state_passing_fwd[_ws] followed by
+ * ssd_chunk_scan_states_fwd (the epoch of opts counts for the first of them; *opts->used_workspace says whether the
+ * chain kernel ran); without `out` and without that kernel there is no place for the passed states: SSD_ERR_SCRATCH
+ * (the library never allocates).
  */
 uint64_t ssd_fused_scan_workspace_bytes(const ssd_dims *dims, int with_out, int chunks_per_item);
 int ssd_fused_chunk_state_passing_scan_fwd(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *C, const ssd_tensor *dt,

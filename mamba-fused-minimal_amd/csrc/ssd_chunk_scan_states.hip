@@ -19,34 +19,13 @@
 // LDS tiles are row-major with the 16-byte piece index XORed with the row number: the loads with LDS destination
 // fix where a lane's 16 bytes land (consecutive lanes, consecutive pieces), so the swizzle is applied on the
 // global side, and the operand reads (16 lanes = 16 rows, same piece) then touch 16 different bank groups.
-#include "ssd_params.h"
-
-#include <utility>
+#include "ssd_tile.h"
 
 namespace ssd {
 
 namespace scan {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
-{
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0x7fffffffLL ? 0x7fffffffLL : bytes),
-                                             0x00020000);
-}
-
-// s_waitcnt immediate that only waits for the vector-memory counter to drop to n (gfx9 field layout)
-constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+using namespace tile;      // register types, pack_bf16, make_rsrc, vmcnt_imm (ssd_tile.h)
 
 // 16 bytes per lane from a buffer straight into LDS: lane l lands at byte 16 * l behind `dst`
 __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t rs, char *dst, int voff, int soff)

@@ -15,6 +15,9 @@
 // are good to about 10 %, which is enough to rank the families; tests/test_cost_model_cpu.py holds the sweep and a
 // second one of 18 other shapes that the fit has not seen, and checks that the family picked is never more than a few
 // per cent slower than the best one the dispatcher could have picked.
+// The constants (microseconds per unit-chunk, per link, the 5 TB/s of the streaming pair) are this one device's: an
+// MI355X with 256 compute units in 8 XCDs of 32 at its steady clocks.  Another compute-unit count rescales them
+// linearly and nothing has been measured at any other value; another part needs its own sweep.
 #pragma once
 
 #include <stdint.h>

@@ -25,26 +25,15 @@
 //
 // Reference semantics: kernels/ssd_chunk_state.py:97-173, kernels/ssd_state_passing.py:27-84,
 // kernels/fused_globalbar.py:16-198 (same math, one launch).
-#include "ssd_params.h"
+#include "ssd_tile.h"
 
 namespace ssd {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+using namespace tile;      // register types, pack_bf16 (ssd_tile.h)
 
 template <int HB> struct FVec;
 template <> struct FVec<4> { typedef f32x4 type; };
 template <> struct FVec<2> { typedef f32x2 type; };
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
-{
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-}
 
 // Workgroup barrier that only orders the LDS reads and writes made by ds instructions: global loads issued
 // earlier -- including the ones that deposit x rows in LDS, which a release fence would wait for -- stay in

@@ -33,36 +33,11 @@ namespace ssd {
 
 namespace quad {
 
-// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
-template <int... I, class F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) { (f(std::integral_constant<int, I>{}), ...); }
-template <int N, class F>
-__device__ __forceinline__ void static_for(F &&f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
+using namespace tile;      // register types, static_for, pack_bf16, make_rsrc, vmcnt_imm, Frag (ssd_tile.h)
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
-{
-    bf16x2 v = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, v);
-}
-
 __device__ __forceinline__ int esize_of(int dt) { return dt == DT_F32 ? 4 : 2; }
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0x7fffffffLL ? 0x7fffffffLL : bytes),
-                                             0x00020000);
-}
-
-// s_waitcnt immediate that only waits for the vector-memory counter to drop to n (gfx9 field layout)
-constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
 // Four consecutive state values of one row -> fp32 / bf16 / f16 destination.  The data registers of a wide store
 // are read out over several cycles after issue; wait states that depend on them keep a following writer of the
@@ -85,8 +60,6 @@ __device__ __forceinline__ void store4(__amdgpu_buffer_rsrc_t rs, int dt, int vo
         asm volatile("s_nop 3" ::"v"(q) : "memory");
     }
 }
-
-struct Frag { uint32_t hi[2][4], lo[2][4]; };
 
 // Steps of B and x kept in LDS (requested ring - 1 steps ahead, into the next chunk at most).  A ring of 8 was
 // measured too (chunk 256 only): same time, so the requests are not what the kernel waits for.

@@ -131,6 +131,18 @@ def test_fused_scan_equals_the_two_calls(ops, oracle):
     assert ops.fused_status() == 0
     assert float((out - out2).abs().max()) <= 1e-4 and float((fin - fin2).abs().max()) <= 1e-4
     assert float((y - y2).abs().max()) <= 2e-3
+    # left to the library, a call that wants `out` as well IS those two calls (the one-launch kernel saves nothing
+    # there): same bits
+    out3, fin3, y3 = ops._fused_chunk_state_state_passing_scan_fwd(*args, Cd, dtd, dAd, torch.float32, initial_states=initd,
+                                                                   y_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert torch.equal(out3, out2) and torch.equal(fin3, fin2) and torch.equal(y3, y2)
+    # ... and without `out` it is the one launch
+    none, fin4, y4 = ops._fused_chunk_state_state_passing_scan_fwd(*args, Cd, dtd, dAd, torch.float32, initial_states=initd,
+                                                                   y_dtype=torch.float32, return_states=False)
+    torch.cuda.synchronize()
+    assert none is None and ops.fused_status() == 0
+    assert float((fin4 - fin2).abs().max()) <= 1e-4 and float((y4 - y2).abs().max()) <= 2e-3
 
 
 def test_fused_scan_falls_back_where_the_chain_kernel_does_not_apply(ops, oracle):
