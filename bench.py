@@ -36,10 +36,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 # inside this script, so the figure is only reported while the sources still hash to the same value; otherwise
 # `roofline.traffic` is null.  The rocprof summaries are kept with the repository.
 MEASURED_TRAFFIC = {
-    "cfg1_mamba2_130m": {"bytes": 114583209, "sources": "0d8ec542dea56218"},
-    "cfg2_mamba2_2p7b": {"bytes": 812754359, "sources": "0d8ec542dea56218"},
-    "cfg3_varlen_packed": {"bytes": 864457874, "sources": "0d8ec542dea56218"},
-    "cfg4_long_grouped": {"bytes": 5366950432, "sources": "0d8ec542dea56218"},
+    "cfg1_mamba2_130m": {"bytes": 114583322, "sources": "0c0365e5b8bd7409"},
+    "cfg2_mamba2_2p7b": {"bytes": 812791003, "sources": "0c0365e5b8bd7409"},
+    "cfg3_varlen_packed": {"bytes": 865284725, "sources": "0c0365e5b8bd7409"},
+    "cfg4_long_grouped": {"bytes": 5363836649, "sources": "0c0365e5b8bd7409"},
 }
 KERNEL_SOURCES = ("ssd_chain_kernel.h", "ssd_chain.hip", "ssd_quad.hip", "ssd_mfma.hip", "ssd_tile.h", "ssd_params.h", "ssd_capi.hip")
 
@@ -205,17 +205,20 @@ def main():
 
     # ... and a kernel with this path's own streams and nothing else: x and B rows in, one fp32 state tile per (state
     # tile, chunk) out, no arithmetic, no chain (ssd_measure_traffic_floor; it overwrites the `out` it is given)
-    mover_ev = None
+    mover_ev = mover_ld_ev = mover_st_ev = None
     if cfg["dtype"] == "bf16" and not args.with_states:
         mv_out = [torch.empty(b, C, H, P, N, device=dev) for _ in range(nsets)]
         mv_fin = torch.empty(b, H, P, N, device=dev)
 
-        def mover(i):
+        def mover(i, part=0):
             s = sets[i % nsets]
-            ssd_amd.measure_traffic_floor(s["B"], s["x"], s["dt"], s["dA_cumsum"], mv_out[i % nsets], mv_fin)
+            ssd_amd.measure_traffic_floor(s["B"], s["x"], s["dt"], s["dA_cumsum"], mv_out[i % nsets], mv_fin, part)
 
         try:
             _, mover_ev = timed(mover, steps_2nd, 3)
+            # ... and each side of its traffic alone: how reads and writes share the memory system
+            _, mover_ld_ev = timed(lambda i: mover(i, 1), steps_2nd, 3)
+            _, mover_st_ev = timed(lambda i: mover(i, 2), steps_2nd, 3)
         except RuntimeError as e:          # a shape the chain kernel does not cover has no such floor
             log(f"[bench] no traffic floor for this workload: {e}")
         del mv_out, mv_fin
@@ -324,6 +327,8 @@ def main():
                      "mover_us": None if mover_ev is None else round(mover_ev * 1e6, 2),
                      "mover_bytes": None if mover_ev is None else b * L * H * P * 2 + d["B"].numel() * 2 + b * C * H * P * N * 4,
                      "frac_of_mover": None if mover_ev is None else round(mover_ev / ev_step, 4),
+                     "mover_loads_us": None if mover_ld_ev is None else round(mover_ld_ev * 1e6, 2),
+                     "mover_stores_us": None if mover_st_ev is None else round(mover_st_ev * 1e6, 2),
                      "kernel_us_cold": round(cold_ev * 1e6, 2), "frac_cold": round(alg_bytes / cold_ev / 1e9 / HBM_PEAK_GBPS, 4)},
         "tflops": round(alg_flops / ev_step / 1e12, 2),
         "mfma_frac_of_bf16_peak": round(2 * alg_flops / ev_step / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),

@@ -395,6 +395,15 @@ int ssd_set_token_split(int waves);
  */
 int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
                               const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, void *stream);
+/*
+ * The same with one side of the traffic left out (no counterpart in the reference either): part 0 = loads and stores
+ * (ssd_measure_traffic_floor), 1 = the loads only (`out` is left alone), 2 = the stores only.  What the three durations
+ * say together is how reads and writes share the device's memory system (bench.py: roofline.mover_loads_us,
+ * roofline.mover_stores_us).  Other values of part: SSD_ERR_SHAPE.
+ */
+int ssd_measure_traffic_floor_part(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt,
+                                   const ssd_tensor *dA_cumsum, const ssd_tensor *out, const ssd_tensor *final_states,
+                                   const ssd_dims *dims, int part, void *stream);
 
 /*
  * Test hook with no counterpart in the reference: the number of XCDs (L2 caches) the LOCAL variant of the ticket /

@@ -756,9 +756,11 @@ int ssd_set_scan_kernel(int kernel)
     return ssd::set_scan_kernel(kernel);
 }
 
-int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
-                              const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, void *stream)
+int ssd_measure_traffic_floor_part(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                                   const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, int part,
+                                   void *stream)
 {
+    if (part < 0 || part > 2) return SSD_ERR_SHAPE;
     Params p;
     int rc = fill_fused(p, x, B, dt, dA_cumsum, nullptr, nullptr, nullptr, out, final_states, dims, 1);
     if (rc) return rc;
@@ -766,7 +768,13 @@ int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ss
     rc = check_device();
     if (rc) return rc;
     const int n_cu = compute_units();
-    return (int)ssd::launch_mover(p, n_cu > 0 ? n_cu : 256, (hipStream_t)stream);
+    return (int)ssd::launch_mover(p, n_cu > 0 ? n_cu : 256, part, (hipStream_t)stream);
+}
+
+int ssd_measure_traffic_floor(const ssd_tensor *x, const ssd_tensor *B, const ssd_tensor *dt, const ssd_tensor *dA_cumsum,
+                              const ssd_tensor *out, const ssd_tensor *final_states, const ssd_dims *dims, void *stream)
+{
+    return ssd_measure_traffic_floor_part(x, B, dt, dA_cumsum, out, final_states, dims, 0, stream);
 }
 
 int ssd_set_chain_xcds(int xcds)

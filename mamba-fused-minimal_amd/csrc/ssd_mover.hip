@@ -9,7 +9,8 @@
 // (ssd_chain.hip): per 32-token step a wave requests its 32 x rows (two requests of 16 rows x 64 bytes) and a quarter of
 // the step's B tile straight into LDS, kDepth steps ahead, and at the end of a chunk stores a tile of 32 x dstate fp32
 // in the fused kernels' store pattern (16 bytes per lane, four adjacent lanes per 64-byte run).  Nothing is read back
-// from LDS and the stored values are a register that holds zeros: `out` is scratch to this kernel.
+// from LDS and the stored values are a register that holds zeros: `out` is scratch to this kernel.  `part` leaves one
+// side out: 1 = the loads only, 2 = the stores only (how the two share the memory system: bench.py times all three).
 #include "ssd_tile.h"
 
 namespace ssd {
@@ -21,7 +22,7 @@ using namespace tile;
 constexpr int kDepth = 7;       // steps of requests in flight per wave, the fused chain kernel's distance
 
 template <int NT, int SPC>
-__global__ void __launch_bounds__(256, 1) mover_kernel(const Params p)
+__global__ void __launch_bounds__(256, 1) mover_kernel(const Params p, const int part)
 {
     constexpr int Q = 32 * SPC, NTW = NT / 4, kPerStep = 2 + NTW, kSlot = kPerStep * 1024;
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -81,39 +82,39 @@ __global__ void __launch_bounds__(256, 1) mover_kernel(const Params p)
     };
     int n = 0;
 #pragma unroll 1
-    for (; n < kDepth; ++n) { request(w_req, s_req, n % (kDepth + 1)); advance_req(); }
+    for (; n < kDepth; ++n) { if (part != 2) request(w_req, s_req, n % (kDepth + 1)); advance_req(); }
     Work w_cur = decode(blockIdx.x);
 #pragma unroll 1
     for (int i = blockIdx.x; i < total; i += gridDim.x) {
 #pragma unroll 1
         for (int s = 0; s < SPC; ++s, ++n) {
-            request(w_req, s_req, n % (kDepth + 1));       // past the end: empty descriptors, nothing fetched
+            if (part != 2) request(w_req, s_req, n % (kDepth + 1));       // past the end: empty descriptors, nothing fetched
             advance_req();
             // the oldest step has landed once only the kDepth newer ones are outstanding (stores issued since count
             // as well, which makes the wait shorter than needed at the first step of a chunk: nothing reads the data)
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(kDepth * kPerStep > 63 ? 63 : kDepth * kPerStep));
             __builtin_amdgcn_s_barrier();                  // the fused kernels share a step's B tile: one barrier per step
         }
-        store_tile(w_cur);
+        if (part != 1) store_tile(w_cur);
         w_cur = decode(i + gridDim.x);
     }
 }
 
 template <int NT, int SPC>
-static hipError_t launch_k(const Params &p, int n_wg, hipStream_t s)
+static hipError_t launch_k(const Params &p, int n_wg, int part, hipStream_t s)
 {
     constexpr int lds = 4 * (kDepth + 1) * (2 + NT / 4) * 1024;
     static std::atomic<uint64_t> configured{0};
     const hipError_t e = ensure_dynamic_lds((const void *)mover_kernel<NT, SPC>, lds, configured);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((mover_kernel<NT, SPC>), dim3(n_wg), dim3(256), lds, s, p);
+    hipLaunchKernelGGL((mover_kernel<NT, SPC>), dim3(n_wg), dim3(256), lds, s, p, part);
     return hipGetLastError();
 }
 
 }  // namespace mover
 
 // p: x, B, out and the sizes of a fused call that the chain kernel covers (chain_supported); `out` is overwritten.
-hipError_t launch_mover(const Params &p_in, int n_cu, hipStream_t s)
+hipError_t launch_mover(const Params &p_in, int n_cu, int part, hipStream_t s)
 {
     Params p = p_in;
     p.n_items = p.batch * p.nheads * (p.headdim / 32);
@@ -121,10 +122,10 @@ hipError_t launch_mover(const Params &p_in, int n_cu, hipStream_t s)
     if (total <= 0) return hipSuccess;
     const int n_wg = (int)(total < n_cu ? total : n_cu);
     const int nt = p.dstate / 16, spc = p.Q / 32;
-    if (nt == 8 && spc == 8) return mover::launch_k<8, 8>(p, n_wg, s);
-    if (nt == 8 && spc == 4) return mover::launch_k<8, 4>(p, n_wg, s);
-    if (nt == 4 && spc == 8) return mover::launch_k<4, 8>(p, n_wg, s);
-    return mover::launch_k<4, 4>(p, n_wg, s);
+    if (nt == 8 && spc == 8) return mover::launch_k<8, 8>(p, n_wg, part, s);
+    if (nt == 8 && spc == 4) return mover::launch_k<8, 4>(p, n_wg, part, s);
+    if (nt == 4 && spc == 8) return mover::launch_k<4, 8>(p, n_wg, part, s);
+    return mover::launch_k<4, 4>(p, n_wg, part, s);
 }
 
 }  // namespace ssd

@@ -215,7 +215,7 @@ __host__ __device__ constexpr int chain_workspace_clear(int i, int n)
 int chain_status_of_header(const int *header);
 int set_chain_xcds(int n);        // 0 = from the device's compute units; a test hook; returns the old value
 // measurement only: the fused call's x / B reads and `out` writes with nothing else (ssd_mover.hip); overwrites p.out
-hipError_t launch_mover(const Params &p, int n_cu, hipStream_t s);
+hipError_t launch_mover(const Params &p, int n_cu, int part, hipStream_t s);
 hipError_t launch_chunk_cumsum(const CumsumParams &p, hipStream_t s);
 bool chunk_cumsum_supported(const CumsumParams &p);
 hipError_t launch_scan_states(const ScanParams &p, hipStream_t s);

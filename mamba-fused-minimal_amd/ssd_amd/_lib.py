@@ -14,7 +14,7 @@ _DTYPES = {torch.float32: SSD_F32, torch.bfloat16: SSD_BF16, torch.float16: SSD_
 
 EXPORTS = ("ssd_version", "ssd_status_string", "ssd_chunk_state_fwd", "ssd_state_passing_fwd",
            "ssd_fused_chunk_state_passing_fwd", "ssd_fused_chunk_state_passing_fwd_ws", "ssd_fused_workspace_bytes", "ssd_fused_workspace_bytes_for",
-           "ssd_fused_workspace_status", "ssd_fused_workspace_status_of", "ssd_set_chain_xcds", "ssd_measure_traffic_floor", "ssd_fused_scan_workspace_bytes", "ssd_fused_chunk_state_passing_scan_fwd", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
+           "ssd_fused_workspace_status", "ssd_fused_workspace_status_of", "ssd_set_chain_xcds", "ssd_measure_traffic_floor", "ssd_measure_traffic_floor_part", "ssd_fused_scan_workspace_bytes", "ssd_fused_chunk_state_passing_scan_fwd", "ssd_fused_chunk_state_passing_fwd_static", "ssd_fused_static_status",
            "ssd_fused_cumsum_chunk_state_passing_fwd", "ssd_fused_cumsum_chunk_state_passing_fwd_ws", "ssd_query_path", "ssd_query_fused_plan", "ssd_chunk_cumsum_fwd", "ssd_chunk_scan_states_fwd", "ssd_set_scan_kernel", "ssd_set_token_split", "ssd_set_segment_chunks")
 
 
@@ -81,6 +81,8 @@ def load():
     lib.ssd_fused_chunk_state_passing_scan_fwd.argtypes = [T] * 10 + [D, ctypes.c_int, ctypes.c_int, ctypes.POINTER(SsdFusedOpts), vp]
     lib.ssd_measure_traffic_floor.restype = ctypes.c_int
     lib.ssd_measure_traffic_floor.argtypes = [T, T, T, T, T, T, D, vp]
+    lib.ssd_measure_traffic_floor_part.restype = ctypes.c_int
+    lib.ssd_measure_traffic_floor_part.argtypes = [T, T, T, T, T, T, D, ctypes.c_int, vp]
     lib.ssd_set_chain_xcds.restype = ctypes.c_int
     lib.ssd_set_chain_xcds.argtypes = [ctypes.c_int]
     lib.ssd_fused_chunk_state_passing_fwd_static.restype = ctypes.c_int

@@ -552,10 +552,11 @@ def set_scan_kernel(kernel):
     return rc
 
 
-def measure_traffic_floor(B, x, dt, dA_cumsum, out, final_states):
+def measure_traffic_floor(B, x, dt, dA_cumsum, out, final_states, part=0):
     """Measurement hook (no counterpart in the reference): enqueues the kernel that moves the bytes of the fused call on
     these tensors -- x and B read, one fp32 state tile per (state tile, chunk) written -- and does nothing else
-    (ssd_measure_traffic_floor).  ``out`` (b,C,H,P,N) fp32 is overwritten with zeros."""
+    (ssd_measure_traffic_floor[_part]).  ``out`` (b,C,H,P,N) fp32 is overwritten with zeros.  ``part``: 0 = loads and
+    stores, 1 = the loads only (``out`` is left alone), 2 = the stores only."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = B.shape
@@ -564,8 +565,9 @@ def measure_traffic_floor(B, x, dt, dA_cumsum, out, final_states):
     dims = _lib.dims_arg(batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks)
     T = _lib.tensor_arg
     with torch.cuda.device(x.device):
-        rc = _lib.load().ssd_measure_traffic_floor(T(x), T(B), T(dt), T(dA_cumsum), T(out), T(final_states), dims, _stream(x))
-    _lib.check(rc, "ssd_measure_traffic_floor")
+        rc = _lib.load().ssd_measure_traffic_floor_part(T(x), T(B), T(dt), T(dA_cumsum), T(out), T(final_states), dims, int(part),
+                                                        _stream(x))
+    _lib.check(rc, "ssd_measure_traffic_floor_part")
 
 
 def set_chain_xcds(xcds):

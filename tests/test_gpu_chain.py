@@ -530,5 +530,15 @@ def test_traffic_floor_kernel_covers_every_output_tile(ops, oracle, kw):
     torch.cuda.synchronize()
     assert int((out != 0).sum()) == 0
     assert bool(torch.isnan(fin).all())
+    # one side of the traffic alone: the loads leave `out` as it is, the stores write all of it
+    out.fill_(float("nan"))
+    ops.measure_traffic_floor(B, x, dt, dA, out, fin, part=1)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(out).all())
+    ops.measure_traffic_floor(B, x, dt, dA, out, fin, part=2)
+    torch.cuda.synchronize()
+    assert int((out != 0).sum()) == 0
+    with pytest.raises(RuntimeError):
+        ops.measure_traffic_floor(B, x, dt, dA, out, fin, part=3)
     with pytest.raises(RuntimeError):                      # fp32 inputs are not the chain kernel's: no floor defined
         ops.measure_traffic_floor(B.float(), x.float(), dt, dA, out, fin)
