@@ -169,10 +169,12 @@ hipError_t launch_chain(const Params &p_in, int n_cu, int mode, hipStream_t s)
     // LOCAL when the units spread evenly over the XCDs and each has a few of its own: producer and consumer of a passed
     // state then share an L2 (no read-back from memory), and an XCD only fetches the B rows of its own units' groups
     // (b=1 L=131072 H=128 G=8: 5.3 GB of HBM traffic instead of 6.5 GB for 4.7 GB algorithmic, 1.15 ms
-    // against 1.17 ms).  With one or
-    // two units per XCD most of its workgroups would sit in one chain.
+    // against 1.17 ms).  With few units per XCD most of its workgroups sit in a few chains, and where all units share
+    // one (batch, group) every XCD fetches all of B anyway: eight units per XCD is where LOCAL starts to pay (five, at
+    // b=1 L=32768 H=80 in 16 packed sequences: 208 us against 204 us with one counter; eight, at b=1 L=131072 H=128 G=8:
+    // 1.065 against 1.068 ms; twenty, at b=4 L=8192 H=80: 179 against 186 us).
     const int fullest = (n_units + p.n_xcd - 1) / p.n_xcd;
-    bool local = mode == 1 || (mode == 0 && n_units >= 4 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
+    bool local = mode == 1 || (mode == 0 && n_units >= 8 * p.n_xcd && (int64_t)fullest * p.n_xcd * 8 <= (int64_t)n_units * 9);
     // Chunks per item: four (what the register file holds parked) unless the estimate says that the compute units
     // end up with too few or too unequal numbers of items that large.  p.n_seg > 0 forces a value.
     const int r = chain_chunks_per_item(p, n_cu, p.n_seg);
