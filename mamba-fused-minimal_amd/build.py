@@ -95,7 +95,7 @@ def build_library(verbose=False, extra_flags=(), jobs=None):
             if name.endswith("gfx950.s"):
                 with open(os.path.join(tmp, name)) as f:
                     text = f.read()
-                findings[src] = isa_check.check_text(text)
+                findings[src] = isa_check.check_text(text) + isa_check.check_operand_reads(text)
                 usage[src] = _resource_usage(text)
         shutil.rmtree(tmp, ignore_errors=True)
     import json

@@ -313,6 +313,52 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         wv[0] = wlo.x; wv[1] = wlo.y; wv[2] = wlo.z; wv[3] = wlo.w;
         wv[4] = whi.x; wv[5] = whi.y; wv[6] = whi.z; wv[7] = whi.w;
     };
+    // Inside the step loop the same reads are inline assembly with a wait of their own, like the B operands below: the
+    // compiler counts LDS operations it has not issued itself as absent, so a wait that it puts in front of the first
+    // use of a read of its own would also wait for every transposing read issued behind that read -- each step would
+    // start by draining the reads that are meant to run ahead of its matrix instructions.  Six instructions: four pairs
+    // of x dwords 256 bytes apart, two quads of weights.
+    struct Ops { u32x2 x[4]; f32x4 w[2]; };
+    constexpr int kOpReads = 6;
+    uint32_t xop_base = (uint32_t)xst_rd, wop_base = (uint32_t)(32 * kg);
+#if defined(__HIP_DEVICE_COMPILE__)
+    xop_base += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)xring;
+    wop_base += (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)wbuf;
+#endif
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wunused-lambda-capture"
+    auto read_ops = [&, xop_base, wop_base](auto sc, int ws, Ops &o) {      // step sc of the chunk whose weights are in slot ws
+        constexpr int s = decltype(sc)::value;
+        constexpr int xo = (s % kRing) * 8, wo = 128 * s;                   // in units of 256 bytes; in bytes
+        const uint32_t wb = wop_base + (uint32_t)(ws * Q * 4);
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("ds_read2st64_b32 %0, %6 offset0:%8 offset1:%9\n\t"
+                     "ds_read2st64_b32 %1, %6 offset0:%10 offset1:%11\n\t"
+                     "ds_read2st64_b32 %2, %6 offset0:%12 offset1:%13\n\t"
+                     "ds_read2st64_b32 %3, %6 offset0:%14 offset1:%15\n\t"
+                     "ds_read_b128 %4, %7 offset:%16\n\t"
+                     "ds_read_b128 %5, %7 offset:%17"
+                     : "=&v"(o.x[0]), "=&v"(o.x[1]), "=&v"(o.x[2]), "=&v"(o.x[3]), "=&v"(o.w[0]), "=&v"(o.w[1])
+                     : "v"(xop_base), "v"(wb), "n"(xo), "n"(xo + 1), "n"(xo + 2), "n"(xo + 3), "n"(xo + 4), "n"(xo + 5),
+                       "n"(xo + 6), "n"(xo + 7), "n"(wo), "n"(wo + 16)
+                     : "memory");
+#else
+        for (int i = 0; i < 4; ++i) o.x[i] = (u32x2){0u, 0u};
+        o.w[0] = o.w[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        (void)wb; (void)xo; (void)wo;
+#endif
+    };
+#pragma clang diagnostic pop
+    // ... valid once no more LDS operations are outstanding than were issued behind them (nc)
+    auto wait_ops = [&](auto nc, Ops &o) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt lgkmcnt(%6) ; operands"
+                     : "+v"(o.x[0]), "+v"(o.x[1]), "+v"(o.x[2]), "+v"(o.x[3]), "+v"(o.w[0]), "+v"(o.w[1])
+                     : "n"(decltype(nc)::value) : "memory");
+#else
+        (void)o;
+#endif
+    };
     // tokens (2q, 2q+1) of headdim row 2*i16 + jp: x * w in fp32, split into bf16 hi + bf16 lo
     auto frag_piece = [&](int q, int jp, const uint32_t (&xr)[8], const float (&wv)[8], Frag &f) {
         const uint32_t r0 = xr[2 * q], r1_ = xr[2 * q + 1];
@@ -919,8 +965,9 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(NTW + (kDist - 2) * (2 + NTW)));
         asm volatile("" ::: "memory");
         uint32_t xr[8]; float wv[8];
-        if (s + 1 < SPC) read_operands(s + 1, ws, xr, wv);
-        else read_operands(0, ws ^ 1, xr, wv);
+        Ops ops;
+        if constexpr (s + 1 < SPC) read_ops(std::integral_constant<int, s + 1>{}, ws, ops);
+        else read_ops(std::integral_constant<int, 0>{}, ws ^ 1, ops);
         if (s == 0 && (cur.r == 0 || (second_late && cur.r == 1)) && threadIdx.x == 0)
             t_new = __hip_atomic_fetch_add(ws_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (s == 0 || s == 2) early_fetch(cur, s);
@@ -939,8 +986,11 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
         __builtin_amdgcn_sched_barrier(0);   // operand reads above, the requests of this step below
         static_for<NT>([&](auto itc) {
             constexpr int it = decltype(itc)::value;
-            // the kAhead - 1 blocks behind this one (two reads each) may still be in flight
-            wait_Bt(std::integral_constant<int, 2 * (kAhead - 1)>{}, blo[it % 4], bhi[it % 4]);
+            // the blocks read behind this one (two reads each) may still be in flight: kAhead - 1 of them, fewer at the
+            // end of a chunk's last step, where the next chunk's first blocks are not read yet
+            constexpr int behind = s + 1 < SPC || NT - 1 - it > kAhead - 1 ? kAhead - 1 : NT - 1 - it;
+            // (the step's operand reads stand behind the first kAhead blocks of its tile and are waited for in iteration 1)
+            wait_Bt(std::integral_constant<int, 2 * behind + (it <= 1 ? kOpReads : 0)>{}, blo[it % 4], bhi[it % 4]);
             const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it % 4].x, blo[it % 4].y, bhi[it % 4].x, bhi[it % 4].y});
             if constexpr (it == NT - kAhead) {
                 // The next read is the first of step + 1's tile: this wave's blocks of it (requested three steps
@@ -965,7 +1015,15 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
             acc[it][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l0, acc[it][0], 0, 0, 0);
             acc[it][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Bt, l1, acc[it][1], 0, 0, 0);
             // next step's x operands, spread over the iterations after the first (their LDS reads, issued at the top
-            // of the step, get the first iteration to arrive)
+            // of the step, get the first iteration to arrive: behind them came the blocks read in iterations 0 and 1)
+            if constexpr (it == 1) {
+                constexpr int after = ((kAhead < NT || s + 1 < SPC) ? 2 : 0) + ((1 + kAhead < NT || s + 1 < SPC) ? 2 : 0);
+                wait_ops(std::integral_constant<int, after>{}, ops);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) xr[j] = ops.x[j >> 1][j & 1];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) wv[j] = ops.w[j >> 2][j & 3];
+            }
             {
                 constexpr int e0 = it == 0 ? 0 : (it - 1) * 8 / (NT - 1), e1 = it == 0 ? 0 : it * 8 / (NT - 1);
 #pragma unroll

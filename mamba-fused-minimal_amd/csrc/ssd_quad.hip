@@ -467,8 +467,10 @@ __global__ void __launch_bounds__(256, 2) quad_kernel(const Params p)
         __builtin_amdgcn_sched_barrier(0);   // stores and operand reads above, the requests of this step below
         static_for<NT>([&](auto itc) {
             constexpr int it = decltype(itc)::value;
-            // the kAhead - 1 blocks behind this one (two reads each) may still be in flight
-            wait_Bt(std::integral_constant<int, 2 * (kAhead - 1)>{}, blo[it % 4], bhi[it % 4]);
+            // the blocks read behind this one (two reads each) may still be in flight: kAhead - 1 of them, fewer at the
+            // end of a chunk's last step, where the next chunk's first blocks are not read yet
+            constexpr int behind = s + 1 < SPC || NT - 1 - it > kAhead - 1 ? kAhead - 1 : NT - 1 - it;
+            wait_Bt(std::integral_constant<int, 2 * behind>{}, blo[it % 4], bhi[it % 4]);
             const bf16x8 Bt = __builtin_bit_cast(bf16x8, (u32x4){blo[it % 4].x, blo[it % 4].y, bhi[it % 4].x, bhi[it % 4].y});
             if constexpr (it == NT - kAhead) {
                 // The next read is the first of step + 1's tile: this wave's blocks of it (requested three steps

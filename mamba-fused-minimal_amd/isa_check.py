@@ -8,6 +8,11 @@ statements -- the copy then holds whatever the register held before the data arr
 Nothing in the source can forbid that, so the generated code is checked: between a transposing read and the first
 matrix instruction that takes its result registers as an operand, no other instruction may read or write them.
 
+The chain kernel reads a step's x and weight operands the same way (`ds_read2st64_b32`, `ds_read_b128` inside an inline
+assembly statement, waited for by the statement whose text ends in "; operands"): between such a read and that wait no
+instruction may touch its result registers either.  Reads of those kinds that the compiler issues itself are its own
+business and are not looked at.
+
 check_text(asm) -> list of findings (empty = clean); check_file(path) the same for a file."""
 import re
 
@@ -60,6 +65,49 @@ def check_text(text, window=600):
     return findings
 
 
+def check_operand_reads(text, window=400):
+    """Inline-assembly x / weight reads: result registers untouched up to the "; operands" wait."""
+    lines = text.split("\n")
+    findings = []
+    kernel = "?"
+    in_asm = False
+    for i, line in enumerate(lines):
+        stripped = line.strip()
+        if stripped.endswith(":") and not stripped.startswith(".") and not stripped.startswith(";"):
+            kernel = stripped[:-1]
+        if stripped.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if stripped.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not in_asm or not (stripped.startswith("ds_read2st64_b32") or stripped.startswith("ds_read_b128")):
+            continue
+        dst = _regs(re.split(r"[ ,]+", stripped)[1])
+        done = False
+        for k in range(i + 1, min(i + window, len(lines))):
+            t = lines[k].strip()
+            if "; operands" in t:
+                done = True
+                break
+            if not t or t[0] in ";." or t.endswith(":"):
+                continue
+            parts = re.split(r"[ ,]+", t)
+            touched = set()
+            for tok in parts[1:]:
+                touched |= _regs(tok)
+            if touched & dst:
+                findings.append({"kernel": kernel, "line": k + 1, "instruction": t, "loaded_at": i + 1,
+                                 "registers": sorted(touched & dst)})
+                done = True
+                break
+        if not done:
+            findings.append({"kernel": kernel, "line": i + 1, "instruction": stripped, "loaded_at": i + 1,
+                             "registers": sorted(dst), "note": "no wait for these operands in sight"})
+    return findings
+
+
 def check_file(path):
     with open(path) as f:
-        return check_text(f.read())
+        text = f.read()
+    return check_text(text) + check_operand_reads(text)

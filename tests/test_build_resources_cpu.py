@@ -95,3 +95,33 @@ _Z6kernelv:
     assert [f["registers"] for f in isa_check.check_text(reused)] == [[12]]
     never_used = clean.replace("\tv_mfma_f32_16x16x32_bf16 a[0:3], v[10:13], v[20:23], a[0:3]\n", "")
     assert len(isa_check.check_text(never_used)) == 1          # overwritten by the v_mov without ever landing in a use
+
+
+def test_the_check_covers_the_operand_reads_of_the_chain_kernel():
+    """x and weight operands of a step are read in inline assembly too and waited for by the statement marked
+    "; operands": nothing may touch their result registers in between, a read without such a wait is reported, and the
+    compiler's own reads of the same kinds are left alone."""
+    import sys
+    sys.path.insert(0, PKG)
+    import isa_check
+    clean = """
+_Z6kernelv:
+	ds_read_b128 v[40:43], v7 offset:64
+	;;#ASMSTART
+	ds_read2st64_b32 v[10:11], v5 offset0:8 offset1:9
+	ds_read_b128 v[12:15], v6 offset:0x80
+	;;#ASMEND
+	v_add_u32_e32 v40, v2, v3
+	v_add_u32_e32 v1, v2, v3
+	;;#ASMSTART
+	s_waitcnt lgkmcnt(4) ; operands
+	;;#ASMEND
+	v_mul_f32_e32 v20, v10, v12
+	s_endpgm
+"""
+    assert isa_check.check_operand_reads(clean) == []
+    moved = clean.replace("v_add_u32_e32 v1, v2, v3", "v_accvgpr_write_b32 a9, v13")
+    found = isa_check.check_operand_reads(moved)
+    assert len(found) == 1 and found[0]["registers"] == [13] and found[0]["kernel"] == "_Z6kernelv"
+    unwaited = clean.replace(" ; operands", "")
+    assert len(isa_check.check_operand_reads(unwaited)) == 2          # both reads: used without their wait
