@@ -279,8 +279,22 @@ __global__ void __launch_bounds__(256, 1) chain_kernel(const Params p)
 #pragma unroll
         for (int t = 0; t < TPL; ++t) m.id[t] = 0;
         if (HAS_SEQ) {
+            // a lane's TPL ids with one load where they are contiguous, aligned and inside the sequence
+            const int32_t *ip = I.sqb + (int64_t)(I.c * Q + TPL * lane) * p.ssq_l;
+            if (p.ssq_l == 1 && (I.c + 1) * Q <= L && ((uintptr_t)(I.sqb + I.c * Q) & 15) == 0) {
+                if constexpr (TPL == 4) {
+                    typedef __attribute__((ext_vector_type(4))) int32_t i32x4;
+                    const i32x4 q = *(const i32x4 *)ip;
+                    m.id[0] = q.x; m.id[1] = q.y; m.id[2] = q.z; m.id[3] = q.w;
+                } else {
+                    typedef __attribute__((ext_vector_type(2))) int32_t i32x2;
+                    const i32x2 q = *(const i32x2 *)ip;
+                    m.id[0] = q.x; m.id[1] = q.y;
+                }
+            } else {
 #pragma unroll
-            for (int t = 0; t < TPL; ++t) m.id[t] = I.sqb[(int64_t)min(I.c * Q + TPL * lane + t, L - 1) * p.ssq_l];
+                for (int t = 0; t < TPL; ++t) m.id[t] = I.sqb[(int64_t)min(I.c * Q + TPL * lane + t, L - 1) * p.ssq_l];
+            }
             m.id_last = I.sqb[(int64_t)(min((I.c + 1) * Q, L) - 1) * p.ssq_l];
             // id of the previous chunk's last token; the recurrence starts from id 0 (kernels/ssd_state_passing.py:68)
             if (I.c > 0) m.id_prev = I.sqb[(int64_t)(I.c * Q - 1) * p.ssq_l];
